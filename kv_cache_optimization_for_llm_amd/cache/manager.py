@@ -82,7 +82,26 @@ class CacheGroup:
             return whole
         step = min(tokens, portion) if portion else tokens
         span = self.spec.window - 1 + step
-        return min(whole, (span + self.page_size - 1) // self.page_size + 1)
+        return min(whole, (span + self.page_size - 1) // self.page_size + 1 + self.kept_blocks)
+
+    @property
+    def kept_blocks(self) -> int:
+        """Leading blocks of a request that a window group never gives back: those that hold one
+        of the first ``keep_first`` positions."""
+        if self.spec.kind != "window" or self.spec.keep_first <= 0:
+            return 0
+        return (self.spec.keep_first + self.page_size - 1) // self.page_size
+
+    def mapped_ranges(self, first_block: int, next_block: int):
+        """The two runs of logical blocks a seat has mapped: the kept head and what the window
+        has not left behind yet (``first_block``: the first block not given back among those that
+        may be)."""
+        head = min(self.kept_blocks, next_block)
+        return (0, head), (max(first_block, head), next_block)
+
+    def held_blocks(self, first_block: int, next_block: int) -> int:
+        (a, b), (c, d) = self.mapped_ranges(first_block, next_block)
+        return (b - a) + (d - c)
 
     def mark_dirty(self, seat: int, lo: int, hi: int) -> None:
         d = self.dirty.get(seat)
@@ -242,8 +261,8 @@ class CacheManager:
         for g in self.groups:
             gi = g.index
             if self.mode == "paged":
-                lo, hi = s.first_block[gi], s.next_block[gi]
-                pages = [int(p) for p in g.table_host[seat, lo:hi] if p >= 0]
+                hi = s.next_block[gi]
+                pages = [int(p) for p in g.table_host[seat, :hi] if p >= 0]
                 g.pool.drop(pages)
                 if hi > 0:
                     g.table_host[seat, :hi] = -1
@@ -274,7 +293,7 @@ class CacheManager:
         s = self.seat(seat)
         if self.mode == "contiguous":
             return self._no_pages
-        return [max(0, g.pages_for(final_len, portion) - (s.next_block[g.index] - s.first_block[g.index]))
+        return [max(0, g.pages_for(final_len, portion) - g.held_blocks(s.first_block[g.index], s.next_block[g.index]))
                 for g in self.groups]
 
     def can_grow(self, seat: int, new_len: int) -> bool:
@@ -348,8 +367,9 @@ class CacheManager:
             if g.spec.kind != "window" or g.spec.window <= 0:
                 continue
             # the next query sits at position >= new_len and reads keys >= new_len - window + 1
+            # (and, whatever the window, the first keep_first positions: their blocks stay)
             keep_from = max(0, new_len - g.spec.window + 1) // self.page_size
-            lo = s.first_block[g.index]
+            lo = max(s.first_block[g.index], g.kept_blocks)
             hi = min(keep_from, s.next_block[g.index])
             if hi > lo:
                 self._before_table_write()
@@ -395,9 +415,10 @@ class CacheManager:
                     continue
                 if self.mode == "paged":
                     lo, hi = s.first_block[g.index], s.next_block[g.index]
-                    if (row[:lo] != -1).any() or (row[hi:] != -1).any() or (row[lo:hi] < 0).any():
+                    (a, b), (c, d) = g.mapped_ranges(lo, hi)
+                    if (row[b:c] != -1).any() or (row[d:] != -1).any() or (row[a:b] < 0).any() or (row[c:d] < 0).any():
                         raise CacheAccountingError(
-                            f"group {g.index}: seat {seat} maps blocks outside [{lo}, {hi})")
+                            f"group {g.index}: seat {seat} maps blocks outside [{a}, {b}) and [{c}, {d})")
                 for p in row[row >= 0]:
                     mapped[int(p)] = mapped.get(int(p), 0) + 1
             if self.mode == "paged":

@@ -67,6 +67,7 @@ FEED_FORWARDS = Registry("feed-forward")
 NORMS = Registry("norm")
 POSITION_ENCODINGS = Registry("position encoding")
 BLOCKS = Registry("block arrangement")
+STREAM_OPS = Registry("operation between layers")
 ROTARY_FREQUENCIES = Registry("rotary frequency rule")     # name -> f(rot_dim, theta, **params) -> fp32 [rot_dim / 2]
 
 
@@ -78,7 +79,9 @@ def register_architecture(name: str, parse_config, build_spec, *, replace: bool 
 
 def architecture_for(config_dict: Mapping[str, Any]) -> Architecture:
     archs = config_dict.get("architectures")
+    if not archs and isinstance(config_dict.get("architecture"), str):
+        archs = [config_dict["architecture"]]           # a single name under the singular key
     if not archs or not isinstance(archs, (list, tuple)):
         raise RegistryError(
-            "config.json has no 'architectures' list; registered: " f"{ARCHITECTURES.names()}")
+            "config.json has no 'architectures' list (or 'architecture' name); registered: " f"{ARCHITECTURES.names()}")
     return ARCHITECTURES.get(archs[0])

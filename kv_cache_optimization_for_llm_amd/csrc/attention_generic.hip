@@ -47,8 +47,8 @@ attention_rowwise_kernel(T *__restrict__ out, const T *__restrict__ q, int q_row
                          const T *__restrict__ k_cache, const T *__restrict__ v_cache,
                          const int *__restrict__ block_table, int max_blocks,
                          const int *__restrict__ tok_seat, const int *__restrict__ tok_pos,
-                         int num_q_heads, int num_kv_heads, int head_dim, int page_size,
-                         float scale, int window) {
+                         int num_q_heads, int num_kv_heads, int head_dim, int value_dim, int page_size,
+                         float scale, int window, int keep_first, const float *__restrict__ sinks) {
     __shared__ float q_s[ATTN_MAX_HEAD_DIM];
     __shared__ float p_s[KVA_WAVE];
     __shared__ long long voff_s[KVA_WAVE];
@@ -68,9 +68,11 @@ attention_rowwise_kernel(T *__restrict__ out, const T *__restrict__ q, int q_row
     float m = -INFINITY, l = 0.f;
     float acc[ATTN_MAX_HEAD_DIM / KVA_WAVE] = {0.f, 0.f, 0.f, 0.f};
 
-    for (int kb = lo / KVA_WAVE; kb <= pos / KVA_WAVE; ++kb) {
+    for (int kb = 0; kb <= pos / KVA_WAVE; ++kb) {
+        // a block with no visible key: behind the window and past the kept first positions
+        if (kb * KVA_WAVE + KVA_WAVE <= lo && kb * KVA_WAVE >= keep_first) continue;
         const int key = kb * KVA_WAVE + lane;
-        const bool valid = key >= lo && key <= pos;
+        const bool valid = key <= pos && (key >= lo || key < keep_first);
         float s = -INFINITY;
         long long row_off = 0;
         if (valid) {
@@ -96,37 +98,45 @@ attention_rowwise_kernel(T *__restrict__ out, const T *__restrict__ q, int q_row
         m = m_new;
         __syncthreads();  // the previous block's p_s / voff_s have been consumed
         p_s[lane] = p;
-        // V is stored transposed inside a page: [page, kv_head, head_dim, page_size]
+        // V is stored transposed inside a page: [page, kv_head, value_dim, page_size]
         voff_s[lane] = valid ? ((long long)bt[key / page_size] * num_kv_heads + kvh) *
-                                       (long long)head_dim * page_size + key % page_size
-                             : 0;
+                                       (long long)value_dim * page_size + key % page_size
+                             : -1;
         __syncthreads();
-        const int first = (kb * KVA_WAVE >= lo) ? 0 : lo - kb * KVA_WAVE;
         const int last = (pos - kb * KVA_WAVE < KVA_WAVE - 1) ? pos - kb * KVA_WAVE : KVA_WAVE - 1;
 #pragma unroll
         for (int c = 0; c < ATTN_MAX_HEAD_DIM / KVA_WAVE; ++c) {
             const int j = lane + c * KVA_WAVE;
-            if (j < head_dim) {
+            if (j < value_dim) {
                 float a = acc[c] * corr;
-                for (int i = first; i <= last; ++i)
-                    a += p_s[i] * to_float(v_cache[voff_s[i] + (long long)j * page_size]);
+                for (int i = 0; i <= last; ++i)
+                    if (voff_s[i] >= 0) a += p_s[i] * to_float(v_cache[voff_s[i] + (long long)j * page_size]);
                 acc[c] = a;
             }
         }
     }
-    T *orow = out + (size_t)t * num_q_heads * head_dim + (size_t)qh * head_dim;
+    if (sinks) {
+        // one more term of the denominator, exp(sink), with no key and no value
+        const float s = sinks[qh], m_new = fmaxf(m, s);
+        const float corr = (m == -INFINITY) ? 0.f : expf(m - m_new);
+        l = l * corr + expf(s - m_new);
+#pragma unroll
+        for (int c = 0; c < ATTN_MAX_HEAD_DIM / KVA_WAVE; ++c) acc[c] *= corr;
+    }
+    T *orow = out + (size_t)t * num_q_heads * value_dim + (size_t)qh * value_dim;
 #pragma unroll
     for (int c = 0; c < ATTN_MAX_HEAD_DIM / KVA_WAVE; ++c) {
         const int j = lane + c * KVA_WAVE;
-        if (j < head_dim) orow[j] = from_float<T>(acc[c] / l);
+        if (j < value_dim) orow[j] = from_float<T>(acc[c] / l);
     }
 }
 
 extern "C" int kva_attention_rowwise(void *out, const void *q, int q_row_stride, const void *k_cache,
                                      const void *v_cache, const int *block_table, int max_blocks,
                                      const int *tok_seat, const int *tok_pos, int tokens,
-                                     int num_q_heads, int num_kv_heads, int head_dim, int page_size,
-                                     float scale, int window, int dtype, hipStream_t stream) {
+                                     int num_q_heads, int num_kv_heads, int head_dim, int value_dim, int page_size,
+                                     float scale, int window, int keep_first, const float *sinks, int dtype,
+                                     hipStream_t stream) {
     KVA_REQUIRE(tokens >= 0 && num_q_heads > 0 && num_kv_heads > 0 && page_size > 0 && max_blocks > 0,
                 "attention: bad sizes");
     KVA_REQUIRE(num_q_heads % num_kv_heads == 0, "attention: %d query heads is not a multiple of %d kv heads",
@@ -136,20 +146,134 @@ extern "C" int kva_attention_rowwise(void *out, const void *q, int q_row_stride,
                 ATTN_MAX_HEAD_DIM);
     KVA_REQUIRE(q_row_stride % 4 == 0, "attention: query row stride %d must be a multiple of 4", q_row_stride);
     KVA_REQUIRE(num_q_heads <= 65535, "attention: too many heads");
-    KVA_REQUIRE(window >= 0, "attention: negative window");
+    KVA_REQUIRE(window >= 0 && keep_first >= 0, "attention: negative window or kept first positions");
+    KVA_REQUIRE(value_dim > 0 && value_dim <= ATTN_MAX_HEAD_DIM, "attention: value size %d must be at most %d",
+                value_dim, ATTN_MAX_HEAD_DIM);
+    if (window == 0) keep_first = 0;
     if (tokens == 0) return KVA_OK;
     dim3 grid(tokens, num_q_heads), block(KVA_WAVE);
     if (dtype == KVA_F32)
         hipLaunchKernelGGL(attention_rowwise_kernel<float>, grid, block, 0, stream, (float *)out,
                            (const float *)q, q_row_stride, (const float *)k_cache,
                            (const float *)v_cache, block_table, max_blocks, tok_seat, tok_pos,
-                           num_q_heads, num_kv_heads, head_dim, page_size, scale, window);
+                           num_q_heads, num_kv_heads, head_dim, value_dim, page_size, scale, window, keep_first, sinks);
     else if (dtype == KVA_BF16)
         hipLaunchKernelGGL(attention_rowwise_kernel<bf16_t>, grid, block, 0, stream, (bf16_t *)out,
                            (const bf16_t *)q, q_row_stride, (const bf16_t *)k_cache,
                            (const bf16_t *)v_cache, block_table, max_blocks, tok_seat, tok_pos,
-                           num_q_heads, num_kv_heads, head_dim, page_size, scale, window);
+                           num_q_heads, num_kv_heads, head_dim, value_dim, page_size, scale, window, keep_first, sinks);
     else KVA_REQUIRE(false, "attention: unsupported dtype %d", dtype);
     KVA_CHECK_LAUNCH("attention_rowwise");
+    return KVA_OK;
+}
+
+// ---- attention over low-rank entries: the plain kernel ----------------------------------------
+//
+// Every token keeps ONE row of `key_dim` = rank + rot elements for all heads: a latent vector of
+// `rank` elements (the value, and - through the query-side product with the key expansion - the
+// unrotated part of the key) followed by the rotated key part.  The query row of a head has the
+// same layout, so score = q . row * scale over all key_dim elements, and the head's output is the
+// probability-weighted sum of the first `rank` elements of the rows; the caller expands it to the
+// head's values.  Rows lie in pages [page_size, key_dim].  Same walk over blocks of 64 keys at
+// absolute positions, window / kept first positions and sink term as the kernel above.
+#define LAT_MAX_KEY_DIM 1280
+#define LAT_MAX_RANK 1024
+
+template <typename T>
+__global__ void __launch_bounds__(KVA_WAVE)
+latent_attention_rowwise_kernel(T *__restrict__ out, const T *__restrict__ q, const T *__restrict__ cache,
+                                const int *__restrict__ block_table, int max_blocks,
+                                const int *__restrict__ tok_seat, const int *__restrict__ tok_pos, int heads,
+                                int rank, int key_dim, int page_size, float scale, int window, int keep_first,
+                                const float *__restrict__ sinks) {
+    __shared__ float q_s[LAT_MAX_KEY_DIM];
+    __shared__ float p_s[KVA_WAVE];
+    __shared__ long long off_s[KVA_WAVE];
+    const int t = blockIdx.x, qh = blockIdx.y, lane = threadIdx.x;
+    const int pos = tok_pos[t];
+    const int *bt = block_table + (size_t)tok_seat[t] * max_blocks;
+    const T *qrow = q + ((size_t)t * heads + qh) * key_dim;
+    for (int j = lane; j < key_dim; j += KVA_WAVE) q_s[j] = to_float(qrow[j]);
+    __syncthreads();
+
+    const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+    float m = -INFINITY, l = 0.f;
+    float acc[LAT_MAX_RANK / KVA_WAVE];
+#pragma unroll
+    for (int c = 0; c < LAT_MAX_RANK / KVA_WAVE; ++c) acc[c] = 0.f;
+
+    for (int kb = 0; kb <= pos / KVA_WAVE; ++kb) {
+        if (kb * KVA_WAVE + KVA_WAVE <= lo && kb * KVA_WAVE >= keep_first) continue;
+        const int key = kb * KVA_WAVE + lane;
+        const bool valid = key <= pos && (key >= lo || key < keep_first);
+        float s = -INFINITY;
+        long long row_off = -1;
+        if (valid) {
+            row_off = ((long long)bt[key / page_size] * page_size + key % page_size) * key_dim;
+            const T *krow = cache + row_off;
+            float dot = 0.f;
+            for (int j = 0; j < key_dim; ++j) dot += q_s[j] * to_float(krow[j]);
+            s = dot * scale;
+        }
+        const float m_new = fmaxf(m, wave_max(s));
+        const float corr = (m == -INFINITY) ? 0.f : expf(m - m_new);
+        const float p = valid ? expf(s - m_new) : 0.f;
+        l = l * corr + wave_sum(p);
+        m = m_new;
+        __syncthreads();
+        p_s[lane] = p;
+        off_s[lane] = row_off;
+        __syncthreads();
+        const int last = (pos - kb * KVA_WAVE < KVA_WAVE - 1) ? pos - kb * KVA_WAVE : KVA_WAVE - 1;
+#pragma unroll
+        for (int c = 0; c < LAT_MAX_RANK / KVA_WAVE; ++c) {
+            const int j = lane + c * KVA_WAVE;
+            if (j < rank) {
+                float a = acc[c] * corr;
+                for (int i = 0; i <= last; ++i)
+                    if (off_s[i] >= 0) a += p_s[i] * to_float(cache[off_s[i] + j]);
+                acc[c] = a;
+            }
+        }
+    }
+    if (sinks) {
+        const float s = sinks[qh], m_new = fmaxf(m, s);
+        const float corr = (m == -INFINITY) ? 0.f : expf(m - m_new);
+        l = l * corr + expf(s - m_new);
+#pragma unroll
+        for (int c = 0; c < LAT_MAX_RANK / KVA_WAVE; ++c) acc[c] *= corr;
+    }
+    T *orow = out + ((size_t)t * heads + qh) * rank;
+#pragma unroll
+    for (int c = 0; c < LAT_MAX_RANK / KVA_WAVE; ++c) {
+        const int j = lane + c * KVA_WAVE;
+        if (j < rank) orow[j] = from_float<T>(acc[c] / l);
+    }
+}
+
+extern "C" int kva_latent_attention_rowwise(void *out, const void *q, const void *cache, const int *block_table,
+                                            int max_blocks, const int *tok_seat, const int *tok_pos, int tokens,
+                                            int heads, int rank, int key_dim, int page_size, float scale,
+                                            int window, int keep_first, const float *sinks, int dtype,
+                                            hipStream_t stream) {
+    KVA_REQUIRE(tokens >= 0 && heads > 0 && heads <= 65535 && page_size > 0 && max_blocks > 0,
+                "latent attention: bad sizes");
+    KVA_REQUIRE(rank > 0 && rank <= LAT_MAX_RANK && key_dim >= rank && key_dim <= LAT_MAX_KEY_DIM,
+                "latent attention: rank %d (at most %d) and row size %d (at most %d) do not fit", rank,
+                LAT_MAX_RANK, key_dim, LAT_MAX_KEY_DIM);
+    KVA_REQUIRE(window >= 0 && keep_first >= 0, "latent attention: negative window or kept first positions");
+    if (window == 0) keep_first = 0;
+    if (tokens == 0) return KVA_OK;
+    dim3 grid(tokens, heads), block(KVA_WAVE);
+    if (dtype == KVA_F32)
+        hipLaunchKernelGGL(latent_attention_rowwise_kernel<float>, grid, block, 0, stream, (float *)out,
+                           (const float *)q, (const float *)cache, block_table, max_blocks, tok_seat, tok_pos,
+                           heads, rank, key_dim, page_size, scale, window, keep_first, sinks);
+    else if (dtype == KVA_BF16)
+        hipLaunchKernelGGL(latent_attention_rowwise_kernel<bf16_t>, grid, block, 0, stream, (bf16_t *)out,
+                           (const bf16_t *)q, (const bf16_t *)cache, block_table, max_blocks, tok_seat, tok_pos,
+                           heads, rank, key_dim, page_size, scale, window, keep_first, sinks);
+    else KVA_REQUIRE(false, "latent attention: unsupported dtype %d", dtype);
+    KVA_CHECK_LAUNCH("latent_attention_rowwise");
     return KVA_OK;
 }

@@ -175,3 +175,14 @@ __device__ inline float block_sum(float v, float *scratch, int nwaves) {
 }
 
 enum KvaDtype { KVA_F32 = 0, KVA_BF16 = 1 };
+
+// Activations of a gated feed-forward, act(gate) * up: silu z / (1 + e^-z), relu, and the tanh
+// form of gelu, 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))).
+enum KvaActivation { KVA_ACT_SILU = 0, KVA_ACT_RELU = 1, KVA_ACT_GELU_TANH = 2 };
+
+__device__ inline float kva_activate(float z, int act) {
+    if (act == KVA_ACT_RELU) return z > 0.f ? z : 0.f;
+    if (act == KVA_ACT_GELU_TANH)
+        return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+    return z * (1.f / (1.f + expf(-z)));
+}

@@ -67,6 +67,7 @@ struct SkinnyArgs {
     void *Y;                 // EPI_PLAIN / EPI_SWIGLU output
     int M, N, K, ldx, ldy;
     int k_waves, out_f32, inter;
+    int act;                 // EPI_SWIGLU: the gate's activation (KvaActivation)
     // row scaling of the input (optional)
     const float *sumsq;
     int sumsq_parts, norm_width;
@@ -609,7 +610,7 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
             for (int i = 0; i < 4; ++i) {
                 if (EPI == EPI_SWIGLU) {
                     const float gt = acc[0][mt][i] * rinv[mt];
-                    v[i] = gt * (1.f / (1.f + expf(-gt))) * (acc[1][mt][i] * rinv[mt]);
+                    v[i] = kva_activate(gt, a.act) * (acc[1][mt][i] * rinv[mt]);
                 } else {
                     v[i] = acc[t][mt][i] * rinv[mt];
                 }
@@ -791,7 +792,11 @@ extern "C" int kva_gemm_skinny(void *Y, const void *X, const void *W, int M, int
                                hipStream_t stream) {
     KVA_REQUIRE(kva_gemm_skinny_supported(M, N, K), "gemm_skinny: M=%d N=%d K=%d not supported "
                 "(1 <= M <= 64, K a multiple of 32)", M, N, K);
+    // (mode 2 carries the gate's activation in the bits above the low four: 2 | activation << 4)
+    const int act = mode >> 4;
+    mode &= 15;
     KVA_REQUIRE(mode >= 0 && mode <= 3, "gemm_skinny: unknown mode %d", mode);
+    KVA_REQUIRE(act >= 0 && act <= KVA_ACT_GELU_TANH && (act == 0 || mode == 2), "gemm_skinny: unknown activation %d", act);
     KVA_REQUIRE(ldx >= K && ldx % 8 == 0, "gemm_skinny: X row stride %d must be a multiple of 8 and >= K", ldx);
     KVA_REQUIRE(mode != 2 || N % 2 == 0, "gemm_skinny: a joined [gate; up] matrix needs an even row count");
     KVA_REQUIRE(sumsq == nullptr || (sumsq_parts >= 1 && norm_width >= 1),
@@ -802,6 +807,7 @@ extern "C" int kva_gemm_skinny(void *Y, const void *X, const void *W, int M, int
     a.X = (const bf16_t *)X; a.W = (const bf16_t *)W; a.Y = Y;
     a.M = M; a.N = N; a.K = K; a.ldx = ldx; a.ldy = ldy; a.k_slices = 1;
     a.inter = mode == 2 ? N / 2 : 0;
+    a.act = act;
     a.out_f32 = mode == 1 ? 1 : 0;
     a.sumsq = sumsq; a.sumsq_parts = sumsq_parts; a.norm_width = norm_width; a.eps = eps;
     a.hidden = (bf16_t *)hidden; a.next_w = next_w; a.next_w_f32 = next_w_f32;

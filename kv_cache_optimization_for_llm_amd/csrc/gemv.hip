@@ -37,6 +37,7 @@ struct GemvArgs {
     // GV_PLAIN / GV_SWIGLU
     void *Y;
     int ldy, out_f32, inter;
+    int act;                     // GV_SWIGLU: the gate's activation (KvaActivation)
     // GV_RESID
     bf16_t *hidden;
     const void *next_w;
@@ -342,7 +343,7 @@ __global__ void __launch_bounds__(64 * GV_WAVES) gemv_kernel(const GemvArgs a) {
             if (cur_active && finishing && col < a.inter) {
                 const float g = gv_pick<RB, M>(acc, 2 * my, my_m), up = gv_pick<RB, M>(acc, 2 * my + 1, my_m);
                 reinterpret_cast<bf16_t *>(a.Y)[(size_t)my_m * a.ldy + col].bits =
-                    float_to_bf16_bits(g * (1.f / (1.f + expf(-g))) * up);
+                    float_to_bf16_bits(kva_activate(g, a.act) * up);
             }
         } else if (EPI == GV_RESID) {
             float sq = 0.f;
@@ -529,7 +530,11 @@ extern "C" int kva_gemv(void *Y, const void *X, const void *W, int M, int N, int
     GemvArgs a = {};
     const int rc = fill_common(a, X, W, M, N, K, ldx, sumsq, sumsq_parts, norm_width, eps);
     if (rc != KVA_OK) return rc;
+    // (mode 2 carries the gate's activation in the bits above the low four: 2 | activation << 4)
+    a.act = mode >> 4;
+    mode &= 15;
     KVA_REQUIRE(mode >= 0 && mode <= 3, "gemv: unknown mode %d", mode);
+    KVA_REQUIRE(a.act >= 0 && a.act <= KVA_ACT_GELU_TANH && (a.act == 0 || mode == 2), "gemv: unknown activation %d", a.act);
     if (mode == 3) {
         KVA_REQUIRE(hidden && scaled_out && sumsq_out, "gemv: the residual epilogue needs hidden, scaled_out and sumsq_out");
         a.hidden = (bf16_t *)hidden; a.next_w = next_w; a.next_w_f32 = next_w_f32;

@@ -1,0 +1,147 @@
+// Kernels around a residual stream that is kept in 32-bit whatever the compute type is:
+// layer norm (weight, no bias) with the pending branch outputs added first and one or two
+// normalised copies written, the join of the stream with a second tensor in front of a product,
+// the gated activation with a choice of activation, and a per-head sigmoid gate.
+//
+// Storage types are run-time codes (KVA_F32 / KVA_BF16) per operand: the stream may be fp32 while
+// the branch outputs and the normalised rows are bf16.  All arithmetic is fp32; sums over a row
+// are taken in a fixed order, so a row's result does not depend on the other rows of the launch.
+#include "common.h"
+#include <math.h>
+
+__device__ inline float ld_as_float(const void *p, int dtype, size_t i) {
+    return dtype == KVA_F32 ? reinterpret_cast<const float *>(p)[i]
+                            : bf16_bits_to_float(reinterpret_cast<const uint16_t *>(p)[i]);
+}
+
+__device__ inline void st_from_float(void *p, int dtype, size_t i, float v) {
+    if (dtype == KVA_F32) reinterpret_cast<float *>(p)[i] = v;
+    else reinterpret_cast<uint16_t *>(p)[i] = float_to_bf16_bits(v);
+}
+
+// One workgroup per output row.  x <- x + d1 + d2 (written back unless rows are gathered), then
+// out_k = (x - mean) / sqrt(var + eps) * w_k with the variance as the mean of squared deviations.
+// With rms != 0 the mean is not taken off: out_k = x / sqrt(mean(x^2) + eps) * w_k.
+__global__ void __launch_bounds__(256)
+layernorm_kernel(void *__restrict__ out1, void *__restrict__ out2, int out_dtype, void *__restrict__ x, int x_dtype,
+                 const void *__restrict__ d1, int d1_dtype, const void *__restrict__ d2, int d2_dtype,
+                 const void *__restrict__ w1, const void *__restrict__ w2, int w_dtype,
+                 const int *__restrict__ row_idx, int width, float eps, int rms) {
+    extern __shared__ float row_s[];
+    __shared__ float red_s[4];
+    const int r = blockIdx.x;
+    const size_t src = (size_t)(row_idx ? row_idx[r] : r) * width, dst = (size_t)r * width;
+    float sum = 0.f;
+    for (int j = threadIdx.x; j < width; j += blockDim.x) {
+        float v = ld_as_float(x, x_dtype, src + j);
+        if (d1) v += ld_as_float(d1, d1_dtype, src + j);
+        if (d2) v += ld_as_float(d2, d2_dtype, src + j);
+        if ((d1 || d2) && !row_idx) {
+            st_from_float(x, x_dtype, src + j, v);
+            v = ld_as_float(x, x_dtype, src + j);       // what the stream holds from now on
+        } else if (d1 || d2) {
+            if (x_dtype == KVA_BF16) v = bf16_bits_to_float(float_to_bf16_bits(v));
+        }
+        row_s[j] = v;
+        sum += v;
+    }
+    float mean = 0.f;
+    if (!rms) mean = block_sum(sum, red_s, blockDim.x / KVA_WAVE) / (float)width;
+    float sq = 0.f;
+    for (int j = threadIdx.x; j < width; j += blockDim.x) {
+        const float dv = row_s[j] - mean;
+        sq += dv * dv;
+    }
+    const float var = block_sum(sq, red_s, blockDim.x / KVA_WAVE) / (float)width;
+    const float inv = 1.0f / sqrtf(var + eps);
+    for (int j = threadIdx.x; j < width; j += blockDim.x) {
+        const float n = (row_s[j] - mean) * inv;
+        st_from_float(out1, out_dtype, dst + j, n * ld_as_float(w1, w_dtype, j));
+        if (out2) st_from_float(out2, out_dtype, dst + j, n * ld_as_float(w2, w_dtype, j));
+    }
+}
+
+extern "C" int kva_layernorm(void *out1, void *out2, int out_dtype, void *x, int x_dtype, const void *d1,
+                             int d1_dtype, const void *d2, int d2_dtype, const void *w1, const void *w2,
+                             int w_dtype, const int *row_idx, int rows, int width, float eps, int rms,
+                             hipStream_t stream) {
+    KVA_REQUIRE(rows >= 0 && width > 0 && width <= 16000, "layernorm: width %d must lie in 1..16000", width);
+    KVA_REQUIRE(out1 && x && w1 && (out2 == nullptr) == (w2 == nullptr), "layernorm: an output without its weight");
+    KVA_REQUIRE(eps >= 0.f, "layernorm: negative eps");
+    if (rows == 0) return KVA_OK;
+    hipLaunchKernelGGL(layernorm_kernel, dim3(rows), dim3(256), (size_t)width * sizeof(float), stream, out1, out2,
+                       out_dtype, x, x_dtype, d1, d1_dtype, d2, d2_dtype, w1, w2, w_dtype, row_idx, width, eps, rms);
+    KVA_CHECK_LAUNCH("layernorm");
+    return KVA_OK;
+}
+
+// out[t] = [ x[t] + d1[t] + d2[t] ; y[t] ] in out's type; x takes the sum (in place).
+__global__ void stream_join_kernel(void *__restrict__ out, int out_dtype, void *__restrict__ x, int x_dtype,
+                                   const void *__restrict__ d1, int d1_dtype, const void *__restrict__ d2,
+                                   int d2_dtype, const void *__restrict__ y, int y_dtype, int wx, int wy) {
+    const size_t t = blockIdx.x;
+    for (int j = threadIdx.x; j < wx; j += blockDim.x) {
+        float v = ld_as_float(x, x_dtype, t * wx + j);
+        if (d1) v += ld_as_float(d1, d1_dtype, t * wx + j);
+        if (d2) v += ld_as_float(d2, d2_dtype, t * wx + j);
+        if (d1 || d2) {
+            st_from_float(x, x_dtype, t * wx + j, v);
+            v = ld_as_float(x, x_dtype, t * wx + j);
+        }
+        st_from_float(out, out_dtype, t * (wx + wy) + j, v);
+    }
+    for (int j = threadIdx.x; j < wy; j += blockDim.x)
+        st_from_float(out, out_dtype, t * (wx + wy) + wx + j, ld_as_float(y, y_dtype, t * wy + j));
+}
+
+extern "C" int kva_stream_join(void *out, int out_dtype, void *x, int x_dtype, const void *d1, int d1_dtype,
+                               const void *d2, int d2_dtype, const void *y, int y_dtype, int rows, int wx, int wy,
+                               hipStream_t stream) {
+    KVA_REQUIRE(rows >= 0 && wx > 0 && wy >= 0, "stream_join: bad sizes");
+    KVA_REQUIRE(out && x && (wy == 0 || y), "stream_join: missing operand");
+    if (rows == 0) return KVA_OK;
+    hipLaunchKernelGGL(stream_join_kernel, dim3(rows), dim3(256), 0, stream, out, out_dtype, x, x_dtype, d1,
+                       d1_dtype, d2, d2_dtype, y, y_dtype, wx, wy);
+    KVA_CHECK_LAUNCH("stream_join");
+    return KVA_OK;
+}
+
+// out[t, i] = act(gu[t, i]) * gu[t, inter + i]
+__global__ void act_mul_kernel(void *__restrict__ out, const void *__restrict__ gu, int dtype, int inter, int act) {
+    const size_t t = blockIdx.y;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= inter) return;
+    const float g = ld_as_float(gu, dtype, t * 2 * inter + i), u = ld_as_float(gu, dtype, t * 2 * inter + inter + i);
+    st_from_float(out, dtype, t * inter + i, kva_activate(g, act) * u);
+}
+
+extern "C" int kva_act_mul(void *out, const void *gate_up, int rows, int inter, int act, int dtype, hipStream_t stream) {
+    KVA_REQUIRE(rows >= 0 && rows <= 65535 && inter > 0, "act_mul: bad sizes");
+    KVA_REQUIRE(act >= KVA_ACT_SILU && act <= KVA_ACT_GELU_TANH, "act_mul: unknown activation %d", act);
+    if (rows == 0) return KVA_OK;
+    hipLaunchKernelGGL(act_mul_kernel, dim3((inter + 255) / 256, rows), dim3(256), 0, stream, out, gate_up, dtype,
+                       inter, act);
+    KVA_CHECK_LAUNCH("act_mul");
+    return KVA_OK;
+}
+
+// x[t, h, :] *= sigmoid(g[t * g_stride + h]) for heads of head_dim elements
+__global__ void head_gate_kernel(void *__restrict__ x, const void *__restrict__ g, int dtype, int heads, int head_dim,
+                                 int g_stride) {
+    const size_t t = blockIdx.x;
+    for (int j = threadIdx.x; j < heads * head_dim; j += blockDim.x) {
+        const float z = ld_as_float(g, dtype, t * g_stride + j / head_dim);
+        const float s = 1.0f / (1.0f + expf(-z));
+        const size_t at = t * heads * head_dim + j;
+        st_from_float(x, dtype, at, ld_as_float(x, dtype, at) * s);
+    }
+}
+
+extern "C" int kva_head_gate(void *x, const void *g, int rows, int heads, int head_dim, int g_stride, int dtype,
+                             hipStream_t stream) {
+    KVA_REQUIRE(rows >= 0 && heads > 0 && head_dim > 0 && g_stride >= heads, "head_gate: bad sizes");
+    if (rows == 0) return KVA_OK;
+    hipLaunchKernelGGL(head_gate_kernel, dim3(rows), dim3(256), 0, stream, x, g, dtype, heads, head_dim, g_stride);
+    KVA_CHECK_LAUNCH("head_gate");
+    return KVA_OK;
+}

@@ -8,7 +8,8 @@ import torch
 
 from .. import parts as _parts  # noqa: F401  (registers the built-in part kinds)
 from . import llama as _llama   # noqa: F401  (registers LlamaForCausalLM)
-from ..config.registry import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, architecture_for)
+from . import gadopel as _gadopel   # noqa: F401  (registers Gadopel)
+from ..config.registry import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, STREAM_OPS, architecture_for)
 from ..models.spec import LayerCall, ModelSpec, TensorSpec
 from ..ops import kernels as K
 from ..parts.base import Block, KVCacheSpec, KVView, MixerContext, NormedRows, StateSpec
@@ -31,10 +32,15 @@ def build_blocks(spec: ModelSpec) -> List[Block]:
     return blocks
 
 
-def model_tensor_specs(spec: ModelSpec, blocks: List[Block], final_norm) -> Dict[str, TensorSpec]:
+def build_stream_ops(spec: ModelSpec) -> list:
+    return [STREAM_OPS.get(ps.kind)(**ps.params) for ps in spec.stream_ops]
+
+
+def model_tensor_specs(spec: ModelSpec, blocks: List[Block], final_norm, stream_ops=()) -> Dict[str, TensorSpec]:
     out: Dict[str, TensorSpec] = {spec.embedding_name: TensorSpec((spec.vocab_size, spec.hidden_size))}
-    for b in blocks:
-        for part in b.parts():
+    groups = [b.parts() for b in blocks] + [tuple(stream_ops)]
+    for parts in groups:
+        for part in parts:
             for name, ts in part.tensor_specs().items():
                 if name in out and out[name] != ts:
                     raise ValueError(f"tensor {name!r} is declared twice with different specs")
@@ -50,7 +56,7 @@ def tensor_specs_for_config(config_dict: Mapping[str, Any]) -> Dict[str, TensorS
     _, spec = spec_for_config(config_dict)
     blocks = build_blocks(spec)
     final_norm = NORMS.get(spec.final_norm.kind)(**spec.final_norm.params)
-    return model_tensor_specs(spec, blocks, final_norm)
+    return model_tensor_specs(spec, blocks, final_norm, build_stream_ops(spec))
 
 
 def resolve_order(spec: ModelSpec) -> List[Tuple[LayerCall, int]]:
@@ -61,6 +67,8 @@ def resolve_order(spec: ModelSpec) -> List[Tuple[LayerCall, int]]:
     for call in spec.order:
         if not 0 <= call.layer < len(spec.layers):
             raise ValueError(f"run order names layer {call.layer}, the model has {len(spec.layers)}")
+        if call.before is not None and not 0 <= call.before < len(spec.stream_ops):
+            raise ValueError(f"run order names stream operation {call.before}, the model has {len(spec.stream_ops)}")
         slot = call.cache
         if slot is None:
             slot, nxt = nxt, nxt + 1
@@ -75,6 +83,13 @@ class Model:
         self.spec, self.dtype, self.device = spec, dtype, torch.device(device)
         self.blocks = build_blocks(spec)
         self.final_norm = NORMS.get(spec.final_norm.kind)(**spec.final_norm.params)
+        self.stream_ops = build_stream_ops(spec)
+        if spec.residual_dtype not in (None, "float32", "bfloat16"):
+            raise ValueError(f"residual_dtype {spec.residual_dtype!r} is not one of None, 'float32', 'bfloat16'")
+        # the type the residual stream is kept in (a model may ask for 32-bit under bf16 products)
+        self.stream_dtype = {None: dtype, "float32": torch.float32, "bfloat16": torch.bfloat16}[spec.residual_dtype]
+        if self.stream_dtype == torch.bfloat16 and dtype == torch.float32:
+            self.stream_dtype = dtype
         self.calls = resolve_order(spec)
         self.embedding: Optional[torch.Tensor] = None
         self.head: Optional[Linear] = None
@@ -123,14 +138,15 @@ class Model:
         results (one layer's are freed while the next one's are made) and fp32 logits at
         ``logit_rows`` places (default: every token).  The engine reserves this much once, and
         leaves it out when it sizes the cache pool from leftover memory."""
-        elem = torch.empty((), dtype=self.dtype).element_size()
+        elem = max(torch.empty((), dtype=self.dtype).element_size(), torch.empty((), dtype=self.stream_dtype).element_size())
         widest = max((sum(part.activation_elements() for part in b.parts()) for b in self.blocks), default=0)
+        widest += max((op.activation_elements() for op in self.stream_ops), default=0)
         rows = int(tokens if logit_rows is None else logit_rows)
         return int(tokens) * (3 * self.spec.hidden_size + 2 * widest) * elem + rows * 4 * self.spec.vocab_size
 
     def graph_safe(self) -> bool:
         """Whether every part may be captured into a HIP graph."""
-        parts = [self.final_norm]
+        parts = [self.final_norm, *self.stream_ops]
         for b in self.blocks:
             parts.append(b)
             parts.extend(b.parts())
@@ -151,13 +167,15 @@ class Model:
 
     # ---- weights
     def tensor_specs(self) -> Dict[str, TensorSpec]:
-        return model_tensor_specs(self.spec, self.blocks, self.final_norm)
+        return model_tensor_specs(self.spec, self.blocks, self.final_norm, self.stream_ops)
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.embedding = tensors[self.spec.embedding_name]
         for b in self.blocks:
             for part in b.parts():
                 part.load(tensors)
+        for op in self.stream_ops:
+            op.load(tensors)
         self.final_norm.load(tensors)
         head = tensors[self.spec.head_name] if self.spec.head_name is not None else self.embedding
         self.head = Linear(head)
@@ -209,12 +227,14 @@ class Model:
         """Runs the batch's tokens through every layer call and returns fp32 logits
         ``[len(batch.logit_rows), vocab]``."""
         T = batch.num_tokens
-        hidden = torch.empty((T, self.spec.hidden_size), dtype=self.dtype, device=self.device)
+        hidden = torch.empty((T, self.spec.hidden_size), dtype=self.stream_dtype, device=self.device)
         delta = None
+        first = None            # the embedding output in the compute type, for operations that read it again
         first_norm = self.blocks[self.calls[0][0].layer].first_norm() if self.calls else self.final_norm
         prep = first_norm.prepared_by_product() if first_norm is not None else None
         if (T <= self.GATHER_PREP_MAX_ROWS and prep is not None and prep[1] == self.spec.hidden_size
                 and self.dtype == torch.bfloat16 and self.embedding.dtype == torch.bfloat16
+                and self.stream_dtype == torch.bfloat16 and not self.stream_ops
                 and self.spec.hidden_size % 8 == 0 and self.spec.embedding_scale == 1.0):
             # a few tokens: the gather prepares the first norm as a product's epilogue would, and
             # the first product finishes it (or one kernel does, as the norm kernel would have)
@@ -227,11 +247,28 @@ class Model:
             K.embed_gather(self.embedding, batch.token_ids, hidden, getattr(batch, "feedback", None))
             if self.spec.embedding_scale != 1.0:
                 K.scale_softcap(hidden, self.spec.embedding_scale)
+            if self.stream_ops:
+                if self.stream_dtype == self.dtype:
+                    first = hidden.clone()
+                else:
+                    first = torch.empty((T, self.spec.hidden_size), dtype=self.dtype, device=self.device)
+                    K.embed_gather(self.embedding, batch.token_ids, first, getattr(batch, "feedback", None))
+                    if self.spec.embedding_scale != 1.0:
+                        K.scale_softcap(first, self.spec.embedding_scale)
         for i, (call, slot) in enumerate(self.calls):
             block = self.blocks[call.layer]
+            if call.before is not None:
+                if isinstance(delta, NormedRows):
+                    raise TypeError("an operation between layers takes the stream, not rows prepared for a norm")
+                pending = () if delta is None else (tuple(delta) if isinstance(delta, (tuple, list)) else (delta,))
+                hidden, delta = self.stream_ops[call.before].forward(hidden, pending, first), None
             # the norm that reads the residual stream after this block
-            next_norm = (self.blocks[self.calls[i + 1][0].layer].first_norm()
-                         if i + 1 < len(self.calls) else self.final_norm)
+            if i + 1 == len(self.calls):
+                next_norm = self.final_norm
+            elif self.calls[i + 1][0].before is not None:
+                next_norm = None            # an operation between the layers reads the stream first
+            else:
+                next_norm = self.blocks[self.calls[i + 1][0].layer].first_norm()
             ctx = MixerContext(batch=batch)
             group = cache.group_of(slot)
             if group is not None:

@@ -56,6 +56,7 @@ class LayerCall:
     layer: int
     cache: Optional[int] = None
     writes_cache: bool = True
+    before: Optional[int] = None        # index into ModelSpec.stream_ops: run on the stream in front of this call
 
 
 @dataclass(frozen=True)
@@ -77,6 +78,11 @@ class ModelSpec:
     logit_scale: float = 1.0
     logit_softcap: float = 0.0
     eos_token_ids: Tuple[int, ...] = ()
+    # Operations on the stream between layers (registry STREAM_OPS), named by LayerCall.before.
+    stream_ops: Tuple[PartSpec, ...] = ()
+    # Type the residual stream is kept in: None = the engine's compute type; "float32" keeps the
+    # stream (and its sums) in 32-bit also where products and activations are bfloat16.
+    residual_dtype: Optional[str] = None
     ignorable_tensors: Tuple[str, ...] = ()   # fnmatch patterns of tensors that may be present unused
 
 

@@ -347,7 +347,7 @@ def rotates_in_kernel(batch, kv, num_q_heads: int, num_kv_heads: int, head_dim: 
 
 def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads: int,
                     num_kv_heads: int, head_dim: int, scale: float, window: int = 0, rope=None,
-                    max_parts: int = 0):
+                    max_parts: int = 0, keep_first: int = 0, sinks=None, value_dim: int = None):
     """Causal GQA attention of the step's tokens over the paged cache.  ``qkv`` is the fused
     projection output ``[T, (nq + 2 nkv) d]`` (or just its Q part) whose first ``nq * d`` columns
     are the (already position-encoded) queries; keys and values are read from ``kv``.
@@ -362,9 +362,23 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
 
     ``max_parts`` > 0: the caller can take the output of one or two decoded tokens as up to so
     many partial results a row (``ops.kernels.AttentionPartials``, returned instead of ``out``,
-    which is then not written) - where the keys are cut that way no merge kernel runs."""
+    which is then not written) - where the keys are cut that way no merge kernel runs.
+
+    ``keep_first`` (with a window: the first so many positions stay visible behind it), ``sinks``
+    (fp32 per query head: one more term exp(sink) in every denominator) and a ``value_dim`` other
+    than ``head_dim`` are taken by the plain kernel only."""
     if kv is None:
         raise K.KernelError("paged_attention: the mixer has no cache view")
+    value_dim = head_dim if value_dim is None else int(value_dim)
+    if window <= 0:
+        keep_first = 0
+    if keep_first > 0 or sinks is not None or value_dim != head_dim:
+        if rope is not None or max_parts:
+            raise K.KernelError("paged_attention: kept first positions, sinks and a value size of its own "
+                                "go with neither rotation inside the kernel nor partial results")
+        return K.attention_rowwise(qkv, qkv.shape[1], out, kv.k_cache, kv.v_cache, kv.block_table,
+                                   batch.tok_seat, batch.positions, num_q_heads, num_kv_heads,
+                                   head_dim, scale, window, keep_first, sinks, value_dim)
     if rope is not None:
         # decoded tokens whose rotation and cache write are still to be done: ``rope`` = (cos, sin)
         # tables or (None, None); only where rotates_in_kernel() said yes

@@ -345,29 +345,231 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, num_q_heads: int, 
         dtype_code(qkv.dtype), _stream()), "rope_kv_write")
 
 
+def check_kv_cache_shapes(what: str, k_cache: torch.Tensor, v_cache: torch.Tensor, num_kv_heads: int,
+                          head_dim: int, value_dim: int) -> int:
+    """:func:`check_cache_shapes` for values of another size than the keys: V pages are
+    ``[kv_heads, value_dim, page_size]``.  Returns the page size."""
+    if value_dim == head_dim:
+        return check_cache_shapes(what, k_cache, v_cache, num_kv_heads, head_dim)
+    if k_cache.dim() != 5 or v_cache.dim() != 4:
+        raise KernelError(f"{what}: the K cache must be 5-D and the V cache 4-D")
+    pages, nkv, chunks, ps, c = k_cache.shape
+    if (nkv, chunks, c) != k_page_shape(num_kv_heads, head_dim) or tuple(v_cache.shape) != (pages, nkv, value_dim, ps):
+        raise KernelError(f"{what}: K cache {tuple(k_cache.shape)} / V cache {tuple(v_cache.shape)} are not "
+                          f"[pages, {num_kv_heads}, {head_dim} / C, page, C] / [pages, {num_kv_heads}, {value_dim}, page]")
+    return int(ps)
+
+
 def attention_rowwise(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_cache: torch.Tensor,
                       v_cache: torch.Tensor, block_table: torch.Tensor, tok_seat: torch.Tensor,
                       tok_pos: torch.Tensor, num_q_heads: int, num_kv_heads: int, head_dim: int,
-                      scale: float, window: int = 0) -> torch.Tensor:
+                      scale: float, window: int = 0, keep_first: int = 0, sinks: Optional[torch.Tensor] = None,
+                      value_dim: Optional[int] = None) -> torch.Tensor:
     """Causal GQA attention of every token over its request's cached keys; ``q`` is a view whose
-    rows are ``q_row_stride`` elements apart (the Q part of a fused QKV buffer)."""
+    rows are ``q_row_stride`` elements apart (the Q part of a fused QKV buffer).  With a
+    ``window`` a query at position i sees key j when ``i - j < window`` or ``j < keep_first``;
+    ``sinks`` (fp32, one per query head) adds ``exp(sink)`` to every softmax denominator;
+    ``value_dim`` is the size of a value where it differs from a key's."""
     tokens = out.shape[0]
-    if out.shape != (tokens, num_q_heads * head_dim):
-        raise KernelError("attention: out must be [T, nq * d]")
-    check_cache_shapes("attention", k_cache, v_cache, num_kv_heads, head_dim)
+    value_dim = head_dim if value_dim is None else int(value_dim)
+    if out.shape != (tokens, num_q_heads * value_dim):
+        raise KernelError("attention: out must be [T, nq * value size]")
+    check_kv_cache_shapes("attention", k_cache, v_cache, num_kv_heads, head_dim, value_dim)
     if block_table.dim() != 2 or tok_seat.shape != (tokens,) or tok_pos.shape != (tokens,):
         raise KernelError("attention: block table [seats, blocks], one seat and position per token")
-    if q.dtype != out.dtype or k_cache.dtype != out.dtype:
+    if q.dtype != out.dtype or k_cache.dtype != out.dtype or v_cache.dtype != out.dtype:
         raise KernelError("attention: q, cache and out must share a dtype")
     if q.data_ptr() % 16 or q_row_stride < num_q_heads * head_dim:
         raise KernelError("attention: q view is misaligned or its stride is too small")
+    if sinks is not None and (sinks.shape != (num_q_heads,) or sinks.dtype != torch.float32):
+        raise KernelError("attention: sinks are fp32, one per query head")
     page_size = k_cache.shape[3]
     check(hip_lib().kva_attention_rowwise(
         _dev(out, "out"), _dev(q, "q", contiguous=False), q_row_stride, _dev(k_cache, "k_cache"),
         _dev(v_cache, "v_cache"), _dev(block_table, "block_table", torch.int32), block_table.shape[1],
         _dev(tok_seat, "tok_seat", torch.int32), _dev(tok_pos, "tok_pos", torch.int32), tokens,
-        num_q_heads, num_kv_heads, head_dim, page_size, float(scale), int(window),
-        dtype_code(out.dtype), _stream()), "attention_rowwise")
+        num_q_heads, num_kv_heads, head_dim, value_dim, page_size, float(scale), int(window), int(keep_first),
+        _opt(sinks, "sinks"), dtype_code(out.dtype), _stream()), "attention_rowwise")
+    return out
+
+
+def latent_attention_rowwise(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor,
+                             tok_seat: torch.Tensor, tok_pos: torch.Tensor, scale: float, window: int = 0,
+                             keep_first: int = 0, sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Causal attention over low-rank entries: ``cache`` ``[pages, page_size, key_dim]`` holds one
+    row per token for all heads, ``q`` ``[T, heads, key_dim]`` rows of the same layout, ``out``
+    ``[T, heads, rank]`` the weighted sums of the rows' first ``rank`` elements."""
+    if q.dim() != 3 or out.dim() != 3 or cache.dim() != 3 or q.shape[:2] != out.shape[:2]:
+        raise KernelError("latent attention: q [T, heads, key_dim], out [T, heads, rank], cache [pages, page, key_dim]")
+    tokens, heads, key_dim = q.shape
+    rank = out.shape[2]
+    if cache.shape[2] != key_dim or rank > key_dim:
+        raise KernelError(f"latent attention: rows of {cache.shape[2]} in the cache, queries of {key_dim}, rank {rank}")
+    if block_table.dim() != 2 or tok_seat.shape != (tokens,) or tok_pos.shape != (tokens,):
+        raise KernelError("latent attention: block table [seats, blocks], one seat and position per token")
+    if q.dtype != out.dtype or cache.dtype != out.dtype:
+        raise KernelError("latent attention: q, cache and out must share a dtype")
+    if sinks is not None and (sinks.shape != (heads,) or sinks.dtype != torch.float32):
+        raise KernelError("latent attention: sinks are fp32, one per head")
+    check(hip_lib().kva_latent_attention_rowwise(
+        _dev(out, "out"), _dev(q, "q"), _dev(cache, "cache"), _dev(block_table, "block_table", torch.int32),
+        block_table.shape[1], _dev(tok_seat, "tok_seat", torch.int32), _dev(tok_pos, "tok_pos", torch.int32),
+        tokens, heads, rank, key_dim, cache.shape[1], float(scale), int(window), int(keep_first),
+        _opt(sinks, "sinks"), dtype_code(out.dtype), _stream()), "latent_attention_rowwise")
+    return out
+
+
+def layernorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor, deltas=(),
+              row_idx: Optional[torch.Tensor] = None, weight2: Optional[torch.Tensor] = None,
+              out2: Optional[torch.Tensor] = None, rms: bool = False) -> torch.Tensor:
+    """``out = (x - mean) / sqrt(var + eps) * weight`` per row (``rms``: without taking the mean
+    off).  ``deltas`` (up to two tensors of x's shape, any of the two storage types) are added to
+    ``x`` first, in place (not written back when ``row_idx`` gathers rows).  ``weight2`` / ``out2``:
+    a second normalised copy with another weight from the same statistics.  ``x`` may be fp32
+    while ``out`` is bf16."""
+    width = x.shape[-1]
+    rows = out.shape[0]
+    deltas = [d for d in deltas if d is not None]
+    if x.dim() != 2 or out.dim() != 2 or out.shape[1] != width or weight.shape != (width,) or len(deltas) > 2:
+        raise KernelError(f"layernorm: shapes x {tuple(x.shape)} weight {tuple(weight.shape)} out {tuple(out.shape)} do not fit")
+    if (row_idx is None and rows != x.shape[0]) or (row_idx is not None and row_idx.shape != (rows,)):
+        raise KernelError("layernorm: one output row per row of x, or per row index")
+    if (weight2 is None) != (out2 is None) or (out2 is not None and (out2.shape != out.shape or out2.dtype != out.dtype
+                                                                      or weight2.shape != (width,) or weight2.dtype != weight.dtype)):
+        raise KernelError("layernorm: the second output needs a weight and out's shape and dtype")
+    for d in deltas:
+        if d.shape != x.shape:
+            raise KernelError("layernorm: a delta must have x's shape")
+    d1 = deltas[0] if deltas else None
+    d2 = deltas[1] if len(deltas) > 1 else None
+    check(hip_lib().kva_layernorm(
+        _dev(out, "out"), _opt(out2, "out2"), dtype_code(out.dtype), _dev(x, "x"), dtype_code(x.dtype),
+        _opt(d1, "delta"), dtype_code(d1.dtype) if d1 is not None else 0,
+        _opt(d2, "delta"), dtype_code(d2.dtype) if d2 is not None else 0,
+        _dev(weight, "weight"), _opt(weight2, "weight2"), dtype_code(weight.dtype),
+        _opt(row_idx, "row_idx", torch.int32), rows, width, float(eps), 1 if rms else 0, _stream()), "layernorm")
+    return out
+
+
+def stream_join(x: torch.Tensor, other: torch.Tensor, out: torch.Tensor, deltas=()) -> torch.Tensor:
+    """``out[t] = [x[t] + deltas ; other[t]]`` in out's type; ``x`` takes the sum in place."""
+    deltas = [d for d in deltas if d is not None]
+    rows, wx = x.shape
+    if other.dim() != 2 or other.shape[0] != rows or out.shape != (rows, wx + other.shape[1]) or len(deltas) > 2 \
+            or any(d.shape != x.shape for d in deltas):
+        raise KernelError(f"stream_join: x {tuple(x.shape)}, other {tuple(other.shape)}, out {tuple(out.shape)} do not fit")
+    d1 = deltas[0] if deltas else None
+    d2 = deltas[1] if len(deltas) > 1 else None
+    check(hip_lib().kva_stream_join(
+        _dev(out, "out"), dtype_code(out.dtype), _dev(x, "x"), dtype_code(x.dtype),
+        _opt(d1, "delta"), dtype_code(d1.dtype) if d1 is not None else 0,
+        _opt(d2, "delta"), dtype_code(d2.dtype) if d2 is not None else 0,
+        _dev(other, "other"), dtype_code(other.dtype), rows, wx, other.shape[1], _stream()), "stream_join")
+    return out
+
+
+ACTIVATIONS = {"silu": 0, "relu": 1, "gelu_tanh": 2}
+
+
+def act_mul(gate_up: torch.Tensor, out: torch.Tensor, activation: str) -> torch.Tensor:
+    """out[t, i] = act(gate_up[t, i]) * gate_up[t, I + i] with ``activation`` one of silu, relu,
+    gelu_tanh (0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))))."""
+    rows, inter = out.shape
+    if activation not in ACTIVATIONS:
+        raise KernelError(f"act_mul: activation {activation!r} is not one of {sorted(ACTIVATIONS)}")
+    if gate_up.shape != (rows, 2 * inter) or gate_up.dtype != out.dtype:
+        raise KernelError(f"act_mul: gate_up {tuple(gate_up.shape)} does not fit out {tuple(out.shape)}")
+    check(hip_lib().kva_act_mul(_dev(out, "out"), _dev(gate_up, "gate_up"), rows, inter, ACTIVATIONS[activation],
+                                dtype_code(out.dtype), _stream()), "act_mul")
+    return out
+
+
+def head_gate(x: torch.Tensor, gates: torch.Tensor, heads: int) -> torch.Tensor:
+    """In place: head h of row t of ``x`` ``[T, heads * d]`` times ``sigmoid(gates[t, h])``; ``gates``
+    is a ``[T, heads]`` view whose rows may be columns of a wider buffer."""
+    rows = x.shape[0]
+    if x.dim() != 2 or x.shape[1] % heads or gates.shape != (rows, heads) or gates.dtype != x.dtype \
+            or gates.stride(1) != 1:
+        raise KernelError(f"head_gate: x {tuple(x.shape)} and gates {tuple(gates.shape)} do not fit {heads} heads")
+    check(hip_lib().kva_head_gate(_dev(x, "x"), _dev(gates, "gates", contiguous=False), rows, heads,
+                                  x.shape[1] // heads, gates.stride(0) if rows > 1 else heads,
+                                  dtype_code(x.dtype), _stream()), "head_gate")
+    return x
+
+
+def qk_encode_cache(qkv: torch.Tensor, positions: torch.Tensor, num_q_heads: int, num_kv_heads: int, head_dim: int,
+                    value_dim: int, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], interleaved: bool,
+                    unit_eps: Optional[float], k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
+                    slot_mapping: Optional[torch.Tensor]) -> None:
+    """Rotates the first ``2 * cos.shape[1]`` elements of every Q and K head of ``qkv``
+    ``[T, nq d + nkv d + nkv value_dim]`` (pair i = elements (2i, 2i + 1) when ``interleaved``, else
+    (i, i + rot / 2)), then - with ``unit_eps`` - divides every head by its root mean square; Q in
+    place, K and the plain V into the paged cache at ``slot_mapping``."""
+    tokens = qkv.shape[0]
+    k_off = num_q_heads * head_dim
+    v_off = k_off + num_kv_heads * head_dim
+    if qkv.dim() != 2 or qkv.shape[1] != v_off + num_kv_heads * value_dim or positions.shape != (tokens,):
+        raise KernelError(f"qk_encode_cache: qkv {tuple(qkv.shape)} is not [T, nq d + nkv d + nkv dv]")
+    rot = 0
+    if cos is not None:
+        if sin is None or cos.shape != sin.shape or cos.dim() != 2:
+            raise KernelError("qk_encode_cache: cos and sin tables must be [positions, rot / 2]")
+        rot = 2 * cos.shape[1]
+    write = k_cache is not None
+    page_size = 0
+    if write:
+        if v_cache is None or slot_mapping is None or slot_mapping.shape != (tokens,) or k_cache.dtype != qkv.dtype \
+                or v_cache.dtype != qkv.dtype:
+            raise KernelError("qk_encode_cache: K and V cache of qkv's dtype and one slot per token are needed")
+        page_size = check_kv_cache_shapes("qk_encode_cache", k_cache, v_cache, num_kv_heads, head_dim, value_dim)
+    check(hip_lib().kva_qk_encode_cache(
+        _dev(qkv, "qkv"), qkv.shape[1], k_off, v_off, _opt(k_cache, "k_cache"), _opt(v_cache, "v_cache"),
+        _opt(cos, "cos", torch.float32), _opt(sin, "sin", torch.float32), _dev(positions, "positions", torch.int32),
+        _opt(slot_mapping if write else None, "slot_mapping", torch.int32), tokens, num_q_heads, num_kv_heads,
+        head_dim, value_dim, rot, 1 if interleaved else 0, -1.0 if unit_eps is None else float(unit_eps),
+        page_size, dtype_code(qkv.dtype), _stream()), "qk_encode_cache")
+
+
+def latent_encode_cache(y: torch.Tensor, kv_off: int, q_lat: torch.Tensor, cache: Optional[torch.Tensor],
+                        norm_weight: torch.Tensor, eps: float, cos: torch.Tensor, sin: torch.Tensor,
+                        positions: torch.Tensor, slot_mapping: Optional[torch.Tensor], heads: int, plain_dim: int,
+                        rank: int, interleaved: bool = False) -> None:
+    """From a projection row ``y[t] = [heads x (plain_dim + rot) | ... rank + rot at kv_off ...]``:
+    the rotated part of every query head goes to ``q_lat[t, h, rank:]``; the entry's first ``rank``
+    elements, RMS-normed with ``norm_weight``, and its rotated last ``rot`` go to row
+    ``slot_mapping[t]`` of ``cache`` ``[pages, page_size, rank + rot]``."""
+    tokens = y.shape[0]
+    rot = 2 * cos.shape[1]
+    if y.dim() != 2 or q_lat.shape != (tokens, heads, rank + rot) or q_lat.dtype != y.dtype or positions.shape != (tokens,):
+        raise KernelError(f"latent_encode_cache: y {tuple(y.shape)} and q_lat {tuple(q_lat.shape)} do not fit")
+    if cos.shape != sin.shape or norm_weight.shape != (rank,):
+        raise KernelError("latent_encode_cache: tables [positions, rot / 2] and a norm weight [rank] are needed")
+    write = cache is not None and slot_mapping is not None
+    if write and (cache.dim() != 3 or cache.shape[2] != rank + rot or cache.dtype != y.dtype
+                  or slot_mapping.shape != (tokens,)):
+        raise KernelError("latent_encode_cache: cache [pages, page_size, rank + rot] of y's dtype, one slot per token")
+    check(hip_lib().kva_latent_encode_cache(
+        _dev(y, "y"), y.shape[1], int(kv_off), _dev(q_lat, "q_lat"), _opt(cache if write else None, "cache"),
+        _dev(norm_weight, "norm_weight"), dtype_code(norm_weight.dtype), float(eps),
+        _dev(cos, "cos", torch.float32), _dev(sin, "sin", torch.float32), _dev(positions, "positions", torch.int32),
+        _opt(slot_mapping if write else None, "slot_mapping", torch.int32), tokens, heads, plain_dim, rank, rot,
+        1 if interleaved else 0, dtype_code(y.dtype), _stream()), "latent_encode_cache")
+
+
+def heads_matmul(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """``out[t, h, :] = w[h] @ x[t, h, :]`` for ``w`` ``[heads, N, K]``.  ``x`` ``[T, heads, K]`` and
+    ``out`` ``[T, heads, N]`` may be views into wider buffers (unit stride along the last axis)."""
+    heads, n, k = w.shape
+    rows = x.shape[0]
+    if x.shape != (rows, heads, k) or out.shape != (rows, heads, n) or x.stride(2) != 1 or out.stride(2) != 1 \
+            or not (x.dtype == w.dtype == out.dtype):
+        raise KernelError(f"heads_matmul: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
+    xr, xh = (x.stride(0), x.stride(1)) if rows > 1 else (max(x.stride(0), (heads - 1) * x.stride(1) + k), x.stride(1))
+    orr, oh = (out.stride(0), out.stride(1)) if rows > 1 else (max(out.stride(0), (heads - 1) * out.stride(1) + n), out.stride(1))
+    if heads == 1:
+        xh, oh = max(xh, k), max(oh, n)
+    check(hip_lib().kva_heads_matmul(_dev(out, "out", contiguous=False), orr, oh, _dev(x, "x", contiguous=False), xr, xh,
+                                     _dev(w, "w"), rows, heads, n, k, dtype_code(x.dtype), _stream()), "heads_matmul")
     return out
 
 
@@ -744,7 +946,7 @@ def gemm_skinny(x: torch.Tensor, w: TiledWeight, out: Optional[torch.Tensor], sw
                 sumsq: Optional[torch.Tensor] = None, norm_width: int = 0, eps: float = 0.0,
                 hidden: Optional[torch.Tensor] = None, next_weight: Optional[torch.Tensor] = None,
                 scaled_out: Optional[torch.Tensor] = None, sumsq_out: Optional[torch.Tensor] = None,
-                x_tiled: bool = False, out_tiled: bool = False):
+                x_tiled: bool = False, out_tiled: bool = False, activation: str = "silu"):
     """out = x @ W^T for at most 64 rows of x (bf16 operands, fp32 accumulation); ``w`` is the
     :class:`TiledWeight` of W.
 
@@ -802,7 +1004,7 @@ def gemm_skinny(x: torch.Tensor, w: TiledWeight, out: Optional[torch.Tensor], sw
     elif out.shape != (m, cols) or (swiglu and out.dtype != torch.bfloat16) \
             or out.dtype not in (torch.bfloat16, torch.float32):
         raise KernelError(f"gemm_skinny: out {tuple(out.shape)} {out.dtype} does not fit")
-    mode = 2 if swiglu else (1 if out_t.dtype == torch.float32 else 0)
+    mode = (2 | ACTIVATIONS[activation] << 4) if swiglu else (1 if out_t.dtype == torch.float32 else 0)     # (the gate's activation rides on mode 2)
     check(lib.kva_gemm_skinny(_dev(out_t, "out"), _dev(x, "x"), _dev(w.data, "w"), m, n, k, k, cols, mode,
                               _opt(sumsq, "sumsq", torch.float32), parts, int(norm_width), float(eps),
                               None, None, 0, None, None, 1 if x_tiled else 0, 1 if out_tiled else 0, _stream()),
@@ -897,7 +1099,8 @@ def gemv_sumsq_parts(n: int, k: int) -> int:
 def gemv(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor], swiglu: bool = False, *,
          sumsq: Optional[torch.Tensor] = None, norm_width: int = 0, eps: float = 0.0,
          hidden: Optional[torch.Tensor] = None, next_weight: Optional[torch.Tensor] = None,
-         scaled_out: Optional[torch.Tensor] = None, sumsq_out: Optional[torch.Tensor] = None):
+         scaled_out: Optional[torch.Tensor] = None, sumsq_out: Optional[torch.Tensor] = None,
+         activation: str = "silu"):
     """out = x @ W^T for one or two rows of x over the plain row-major bf16 weight ``w`` [N, K]
     (fp32 accumulation).  The options are :func:`gemm_skinny`'s: ``swiglu`` for a joined
     ``[gate; up]`` matrix, ``sumsq`` to finish the input's norm, ``hidden`` / ``next_weight`` /
@@ -932,7 +1135,7 @@ def gemv(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor], swiglu: 
     if out.shape != (m, cols) or (swiglu and out.dtype != torch.bfloat16) \
             or out.dtype not in (torch.bfloat16, torch.float32) or not out.is_contiguous():
         raise KernelError(f"gemv: out {tuple(out.shape)} {out.dtype} does not fit")
-    mode = 2 if swiglu else (1 if out.dtype == torch.float32 else 0)
+    mode = (2 | ACTIVATIONS[activation] << 4) if swiglu else (1 if out.dtype == torch.float32 else 0)
     check(lib.kva_gemv(_dev(out, "out"), _dev(x, "x", contiguous=False), _dev(w, "w"), m, n, k, x.stride(0), cols, mode, *norm,
                        None, None, 0, None, None, _stream()), "gemv")
     return out

@@ -41,9 +41,13 @@ class EncodedQKV:
     ROTATE_LATER_ELEMENTS = 1 << 24
 
     def __init__(self, linear: Linear, position, hidden_size: int, num_heads: int, num_kv_heads: int,
-                 head_dim: int):
+                 head_dim: int, value_dim: Optional[int] = None, rotate_later: bool = True):
         self.linear, self.position = linear, position
+        # False: the attention call that follows has options the kernel that rotates inside lacks
+        self.rotate_later = bool(rotate_later)
         self.hidden_size, self.num_heads, self.num_kv_heads, self.head_dim = hidden_size, num_heads, num_kv_heads, head_dim
+        # values of another size than the keys: only the encoding's own kernel lays such rows out
+        self.value_dim = int(head_dim if value_dim is None else value_dim)
         self.pending_rotation = None          # set by a call that left encoding and cache write to the attention kernel
 
     def __call__(self, x, batch, kv):
@@ -55,13 +59,18 @@ class EncodedQKV:
         self.pending_rotation = None
         tables, rows = None, x.shape[0]
         kernel = self.linear.fused_kernel(rows, x.dtype, rotated=True)
+        if self.value_dim != self.head_dim:
+            qkv = self.linear(x)
+            self.position.apply_and_cache(qkv, batch.positions, self.num_heads, self.num_kv_heads,
+                                          self.head_dim, kv, value_dim=self.value_dim)
+            return qkv
         if kernel == Linear.GEMV and not K.gemv_qkv_rope_supported(rows, self.hidden_size, self.head_dim):
             kernel = Linear.FEW_ROWS if self.linear.tiled is not None else None
         if kernel == Linear.FEW_ROWS and not K.gemm_skinny_qkv_rope_supported(rows, self.hidden_size, self.head_dim):
             kernel = None
         if (kernel == Linear.FEW_ROWS and rows > SKINNY_MAX_ROWS
                 and (rows <= self.ROTATE_LATER_ROWS or self.linear.weight.numel() <= self.ROTATE_LATER_ELEMENTS)
-                and attn_ops.rotates_in_kernel(batch, kv, self.num_heads, self.num_kv_heads, self.head_dim, x.dtype)):
+                and self.rotate_later and attn_ops.rotates_in_kernel(batch, kv, self.num_heads, self.num_kv_heads, self.head_dim, x.dtype)):
             kernel = None
         if kernel is not None:
             tables = self.position.rotate_half_tables(x.device, self.head_dim)
@@ -70,7 +79,7 @@ class EncodedQKV:
             # decoded tokens only: rotation and cache write go into the attention kernel, which
             # takes the product as it is (one launch less per layer where the product is the library's)
             later = self.position.rotate_half_tables(x.device, self.head_dim)
-            if later is not None and attn_ops.rotates_in_kernel(batch, kv, self.num_heads, self.num_kv_heads,
+            if later is not None and self.rotate_later and attn_ops.rotates_in_kernel(batch, kv, self.num_heads, self.num_kv_heads,
                                                                 self.head_dim, qkv.dtype):
                 self.pending_rotation = later
                 return qkv
@@ -97,43 +106,55 @@ class GQAAttention(Mixer):
     graph_safe = True
 
     def __init__(self, prefix: str, *, hidden_size: int, num_heads: int, num_kv_heads: int,
-                 head_dim: int, scale: float, position: PartSpec, window: int = 0):
+                 head_dim: int, scale: float, position: PartSpec, window: int = 0, keep_first: int = 0,
+                 value_dim: Optional[int] = None, tensor_names: Optional[Dict[str, str]] = None):
+        """``window`` > 0: a query at position i sees key j only when ``i - j < window`` or
+        ``j < keep_first`` (the first positions of a request stay visible, at their true places).
+        ``value_dim``: the size of a value head where it is not ``head_dim``.  ``tensor_names``
+        maps ``q``, ``k``, ``v``, ``o`` to the names (behind ``prefix``) of the four matrices."""
         super().__init__(prefix)
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads is not a multiple of {num_kv_heads} kv heads")
         self.hidden_size, self.num_heads, self.num_kv_heads = hidden_size, num_heads, num_kv_heads
         self.head_dim, self.scale, self.window = head_dim, float(scale), int(window)
+        self.keep_first = int(keep_first) if self.window > 0 else 0
+        self.value_dim = int(head_dim if value_dim is None else value_dim)
+        names = dict(q="q_proj.weight", k="k_proj.weight", v="v_proj.weight", o="o_proj.weight")
+        names.update(tensor_names or {})
+        self.names = {key: prefix + name for key, name in names.items()}
         self.position = POSITION_ENCODINGS.get(position.kind)(**position.params)
         self.qkv: Optional[EncodedQKV] = None
         self.o: Optional[Linear] = None
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
-        p, d = self.prefix, self.head_dim
+        n, d, dv = self.names, self.head_dim, self.value_dim
         return {
-            p + "q_proj.weight": TensorSpec((self.num_heads * d, self.hidden_size)),
-            p + "k_proj.weight": TensorSpec((self.num_kv_heads * d, self.hidden_size)),
-            p + "v_proj.weight": TensorSpec((self.num_kv_heads * d, self.hidden_size)),
-            p + "o_proj.weight": TensorSpec((self.hidden_size, self.num_heads * d)),
+            n["q"]: TensorSpec((self.num_heads * d, self.hidden_size)),
+            n["k"]: TensorSpec((self.num_kv_heads * d, self.hidden_size)),
+            n["v"]: TensorSpec((self.num_kv_heads * dv, self.hidden_size)),
+            n["o"]: TensorSpec((self.hidden_size, self.num_heads * dv)),
         }
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
-        p = self.prefix
-        q, k, v = (tensors[p + n + "_proj.weight"] for n in "qkv")
+        q, k, v = (tensors[self.names[n]] for n in "qkv")
         if not (q.dtype == k.dtype == v.dtype):
-            raise ValueError(f"{p}: q/k/v projection weights are stored in different dtypes")
+            raise ValueError(f"{self.prefix}: q/k/v projection weights are stored in different dtypes")
         self.qkv = EncodedQKV(Linear(torch.cat([q, k, v], dim=0)), self.position, self.hidden_size,
-                              self.num_heads, self.num_kv_heads, self.head_dim)
-        self.o = Linear(tensors[p + "o_proj.weight"])
+                              self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim,
+                              rotate_later=self.keep_first == 0)
+        self.o = Linear(tensors[self.names["o"]])
 
     def kv_cache_spec(self) -> KVCacheSpec:
         return attention_cache_spec(self.num_kv_heads, self.head_dim,
-                                    kind="window" if self.window > 0 else "full", window=self.window)
+                                    kind="window" if self.window > 0 else "full", window=self.window,
+                                    value_dim=self.value_dim, keep_first=self.keep_first)
 
     fuses_tail = True
 
     def activation_elements(self) -> int:
         # the joined projection, the attention output and the output projection
-        return (2 * self.num_heads + 2 * self.num_kv_heads) * self.head_dim + self.hidden_size
+        return ((self.num_heads + self.num_kv_heads) * (self.head_dim + self.value_dim)
+                + self.hidden_size)
 
     def forward(self, x, ctx: MixerContext, tail: Optional[BranchTail] = None):
         """``x`` may be NormedRows (the input norm is then finished inside the QKV product); with
@@ -141,14 +162,15 @@ class GQAAttention(Mixer):
         norm when the shapes allow, and NormedRows are returned instead of the plain output."""
         batch, kv = ctx.batch, ctx.kv
         qkv = self.qkv(x, batch, kv)
-        out = torch.empty((x.shape[0], self.num_heads * self.head_dim), dtype=x.dtype, device=x.device)
+        out = torch.empty((x.shape[0], self.num_heads * self.value_dim), dtype=x.dtype, device=x.device)
         # an output projection that adds the key ranges' partial results up itself (one or two
         # decoded tokens) is told so: the attention kernel may then leave them unmerged
+        plain = self.keep_first == 0 and self.value_dim == self.head_dim
         max_parts = self.o.takes_attention_partials(x.shape[0], x.dtype, tail, self.head_dim) \
-            if self.qkv.pending_rotation is None else 0
+            if self.qkv.pending_rotation is None and plain else 0
         out = attn_ops.paged_attention(qkv, out, kv, batch, self.num_heads, self.num_kv_heads,
                                        self.head_dim, self.scale, self.window, rope=self.qkv.pending_rotation,
-                                       max_parts=max_parts)
+                                       max_parts=max_parts, keep_first=self.keep_first, value_dim=self.value_dim)
         if tail is not None:
             fused = self.o.into_residual(out, tail)
             if fused is not None:

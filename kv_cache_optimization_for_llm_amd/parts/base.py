@@ -70,12 +70,14 @@ class KVCacheSpec:
     """Paged storage one mixer call needs: the arrays it keeps per token (names, per-token
     shapes, layout inside a page) and which positions stay.  ``kind`` is ``"full"`` (every
     position stays) or ``"window"`` (only the last ``window`` positions are ever read, pages
-    behind them are given back).  The cache manager allocates from this description and the
-    engine sizes the pool from it; neither knows what the arrays mean."""
+    behind them are given back; with ``keep_first`` the first so many positions of a request stay
+    readable as well, whatever the window).  The cache manager allocates from this description and
+    the engine sizes the pool from it; neither knows what the arrays mean."""
 
     arrays: Tuple[CacheArray, ...]
     kind: str = "full"
     window: int = 0
+    keep_first: int = 0
 
     def __post_init__(self):
         names = [a.name for a in self.arrays]
@@ -89,15 +91,19 @@ class KVCacheSpec:
                    for a in self.arrays)
 
 
-def attention_cache_spec(num_kv_heads: int, head_dim: int, kind: str = "full", window: int = 0) -> KVCacheSpec:
+def attention_cache_spec(num_kv_heads: int, head_dim: int, kind: str = "full", window: int = 0,
+                         value_dim: Optional[int] = None, keep_first: int = 0) -> KVCacheSpec:
     """Keys and values of ``num_kv_heads`` heads of ``head_dim``, as the attention kernels here
     read them: K pages ``[kv_heads, head_dim / C, page_size, C]`` (a key in chunks of C = 8
     elements, 4 where the head size is no multiple of 8; the chunks of a page's keys next to each
     other, so that a wavefront's matrix-core operand is one run of bytes), V pages transposed
-    ``[kv_heads, head_dim, page_size]``."""
+    ``[kv_heads, value_dim, page_size]`` (``value_dim``: the size of a value where it is not the
+    key's)."""
     chunk = 4 if head_dim % 8 else 8
+    value_dim = int(head_dim if value_dim is None else value_dim)
     return KVCacheSpec((CacheArray("k", (int(num_kv_heads), int(head_dim) // chunk, chunk), token_axis=2),
-                        CacheArray("v", (int(num_kv_heads), int(head_dim)), token_axis=2)), kind, window)
+                        CacheArray("v", (int(num_kv_heads), value_dim), token_axis=2)), kind, window,
+                       int(keep_first) if kind == "window" else 0)
 
 
 @dataclass(frozen=True)

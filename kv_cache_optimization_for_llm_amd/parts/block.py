@@ -46,3 +46,44 @@ class PreNormBlock(Block):
         else:
             f = self.feed_forward.forward(x, ctx)
         return hidden, f
+
+
+@BLOCKS.register("parallel")
+class ParallelBlock(Block):
+    """Both branches read the same stream: ``h += mixer(norm_m(h)) + ffn(norm_f(h))``.
+
+    The two branch outputs are handed on as ``delta`` (a tuple) and added by whatever reads the
+    stream next - this block's own norm pass, the next block's, the final norm or an operation
+    between layers - in one pass over the stream, in the stream's own type (an fp32 stream stays
+    fp32 whatever the branches compute in).  When both norms are of one form with the same width
+    and eps (``forward_pair``), one pass writes both normalised copies.  A layer without a
+    feed-forward (``"none"``) names only the ``"mixer"`` norm."""
+
+    graph_safe = True
+    NORM_NAMES = ("mixer", "feed_forward")
+
+    def __init__(self, mixer, feed_forward, norms):
+        self.has_ffn = not getattr(feed_forward, "absent", False)
+        if not self.has_ffn:
+            self.NORM_NAMES = ("mixer",)
+        super().__init__(mixer, feed_forward, norms)
+        self.mixer_norm = self.norms["mixer"]
+        self.ffn_norm = self.norms.get("feed_forward")
+
+    def first_norm(self) -> Optional[Norm]:
+        return None             # the stream is handed over as it is, with its pending branch outputs
+
+    def forward(self, hidden: torch.Tensor, delta, ctx: MixerContext, next_norm: Optional[Norm] = None):
+        if isinstance(delta, NormedRows):
+            raise TypeError("a parallel block takes the stream and plain branch outputs, not prepared rows")
+        pair = getattr(self.mixer_norm, "forward_pair", None)
+        if self.has_ffn and pair is not None and type(self.ffn_norm) is type(self.mixer_norm) \
+                and (self.ffn_norm.width, self.ffn_norm.eps) == (self.mixer_norm.width, self.mixer_norm.eps):
+            xm, xf = pair(self.ffn_norm, hidden, delta=delta)
+        else:
+            xm = self.mixer_norm.forward(hidden, delta=delta)        # adds the pending outputs to the stream
+            xf = self.ffn_norm.forward(hidden) if self.has_ffn else None
+        a = self.mixer.forward(xm, ctx)
+        if not self.has_ffn:
+            return hidden, a
+        return hidden, (a, self.feed_forward.forward(xf, ctx))

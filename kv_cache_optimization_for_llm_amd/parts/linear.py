@@ -120,8 +120,8 @@ class Linear:
             return None
         return K.gemm_skinny_partials(x, self.tiled)
 
-    def gated(self, x, out) -> None:
-        """``out`` = silu(x gate^T) * (x up^T) for a joined [gate; up] weight whose rows
+    def gated(self, x, out, activation: str = "silu") -> None:
+        """``out`` = act(x gate^T) * (x up^T) for a joined [gate; up] weight whose rows
         :meth:`fusable` accepts; ``out`` is [rows, out_features / 2] or, for the few-rows kernel,
         an ``ops.kernels.TiledRows`` of that size."""
         norm = {}
@@ -129,9 +129,10 @@ class Linear:
             norm = dict(sumsq=x.sumsq, norm_width=x.width, eps=x.eps)
             x = x.scaled
         if self.fused_kernel(x.shape[0], x.dtype) == self.GEMV:
-            K.gemv(x, self.weight, out, swiglu=True, **norm)
+            K.gemv(x, self.weight, out, swiglu=True, activation=activation, **norm)
         else:
-            K.gemm_skinny(x, self.tiled, out, swiglu=True, out_tiled=isinstance(out, K.TiledRows), **norm)
+            K.gemm_skinny(x, self.tiled, out, swiglu=True, out_tiled=isinstance(out, K.TiledRows),
+                          activation=activation, **norm)
 
     def __call__(self, x, out: Optional[torch.Tensor] = None,
                  out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:

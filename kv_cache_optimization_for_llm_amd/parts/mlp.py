@@ -1,7 +1,10 @@
-"""SwiGLU feed-forward: ``down( silu(gate(x)) * up(x) )``, no biases
+"""Gated feed-forward: ``down( act(gate(x)) * up(x) )``, no biases; SwiGLU is ``act = silu``
 (reference: ``base/src/engine.cu:780-858``, ``siluKernel`` ``base/src/kernels.cu:45-52``).
 
 Gate and up matrices are joined at load time into one ``[2 * intermediate, hidden]`` matrix.
+The activation is a parameter (``silu``, ``relu``, ``gelu_tanh``); the products that apply it in
+their epilogue exist for ``silu``, another activation runs as its own kernel behind the joined
+product.  ``"none"`` is the feed-forward of a layer that has none.
 """
 from __future__ import annotations
 
@@ -16,31 +19,50 @@ from .base import BranchTail, FeedForward, MixerContext, NormedRows
 from .linear import Linear
 
 
+@FEED_FORWARDS.register("none")
+class NoFeedForward(FeedForward):
+    """A layer without a feed-forward branch: the block skips it."""
+
+    graph_safe = True
+    absent = True
+
+    def __init__(self, prefix: str = "", **_ignored):
+        super().__init__(prefix)
+
+    def forward(self, x, ctx: MixerContext, tail: Optional[BranchTail] = None):
+        raise RuntimeError("a layer without a feed-forward has no branch to run")
+
+
+@FEED_FORWARDS.register("gated")
 @FEED_FORWARDS.register("swiglu")
 class SwiGLU(FeedForward):
     graph_safe = True
 
-    def __init__(self, prefix: str, *, hidden_size: int, intermediate_size: int):
+    def __init__(self, prefix: str, *, hidden_size: int, intermediate_size: int, activation: str = "silu",
+                 tensor_names: Optional[Dict[str, str]] = None):
+        """``tensor_names`` maps ``gate``, ``up``, ``down`` to the matrices' names behind ``prefix``."""
         super().__init__(prefix)
+        if activation not in K.ACTIVATIONS:
+            raise ValueError(f"activation {activation!r} is not one of {sorted(K.ACTIVATIONS)}")
+        self.activation = activation
+        names = dict(gate="gate_proj.weight", up="up_proj.weight", down="down_proj.weight")
+        names.update(tensor_names or {})
+        self.names = {key: prefix + name for key, name in names.items()}
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
         self.gate_up: Optional[Linear] = None
         self.down: Optional[Linear] = None
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
-        p, h, i = self.prefix, self.hidden_size, self.intermediate_size
-        return {
-            p + "gate_proj.weight": TensorSpec((i, h)),
-            p + "up_proj.weight": TensorSpec((i, h)),
-            p + "down_proj.weight": TensorSpec((h, i)),
-        }
+        n, h, i = self.names, self.hidden_size, self.intermediate_size
+        return {n["gate"]: TensorSpec((i, h)), n["up"]: TensorSpec((i, h)), n["down"]: TensorSpec((h, i))}
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         p = self.prefix
-        g, u = tensors[p + "gate_proj.weight"], tensors[p + "up_proj.weight"]
+        g, u = tensors[self.names["gate"]], tensors[self.names["up"]]
         if g.dtype != u.dtype:
             raise ValueError(f"{p}: gate and up projection weights are stored in different dtypes")
         self.gate_up = Linear(torch.cat([g, u], dim=0), halves=2)
-        self.down = Linear(tensors[p + "down_proj.weight"])
+        self.down = Linear(tensors[self.names["down"]])
 
     fuses_tail = True
 
@@ -63,9 +85,11 @@ class SwiGLU(FeedForward):
             act = torch.empty((rows, self.intermediate_size), dtype=x.dtype, device=x.device)
         if up_kernel is not None:
             # activation fused into the product; an unfinished input norm is finished there too
-            self.gate_up.gated(x, act)
-        else:
+            self.gate_up.gated(x, act, self.activation)
+        elif self.activation == "silu":
             K.silu_mul(self.gate_up(x), act)
+        else:
+            K.act_mul(self.gate_up(x), act, self.activation)
         if tail is not None:
             fused = self.down.into_residual(act, tail)
             if fused is not None:

@@ -45,3 +45,54 @@ class RMSNorm(Norm):
         if isinstance(delta, K.PartialSums) and (x.dtype != torch.bfloat16 or self.width % 8):
             delta = delta.materialize()
         return K.rmsnorm(x, self.weight, self.eps, out, delta=delta, row_idx=row_idx)
+
+
+@NORMS.register("layernorm")
+class LayerNorm(Norm):
+    """``y = (x - mean) / sqrt(var + eps) * w`` with the variance as the mean of the squared
+    deviations; a weight, no bias.  Statistics are fp32.  The rows it reads may be an fp32 stream
+    while it writes ``out_dtype`` rows (the type the products behind it take).  ``delta`` may be one
+    branch output or a tuple of two: they are added to ``x`` in place first.  ``forward_pair``
+    writes two normalised copies, this norm's and a ``twin``'s (same width and eps, another
+    weight), from one pass and one set of statistics."""
+
+    graph_safe = True
+
+    def __init__(self, prefix: str, *, width: int, eps: float, weight_name: str = "weight",
+                 out_dtype: Optional[str] = None):
+        super().__init__(prefix)
+        self.width, self.eps = int(width), float(eps)
+        self.weight_name = prefix + weight_name
+        self.out_dtype = {None: None, "bfloat16": torch.bfloat16, "float32": torch.float32}[out_dtype]
+        self.weight: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return {self.weight_name: TensorSpec((self.width,), init="norm", role="vector")}
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.weight = tensors[self.weight_name].contiguous()
+
+    def activation_elements(self) -> int:
+        return self.width
+
+    @staticmethod
+    def _deltas(delta):
+        if delta is None:
+            return ()
+        return tuple(delta) if isinstance(delta, (tuple, list)) else (delta,)
+
+    def _out(self, x, row_idx):
+        rows = x.shape[0] if row_idx is None else row_idx.shape[0]
+        # the products behind a norm take the weights' type; a 32-bit stream of a bf16 model is normalised into bf16
+        return torch.empty((rows, self.width), dtype=self.out_dtype or self.weight.dtype, device=x.device)
+
+    def forward(self, x, out=None, delta=None, row_idx=None):
+        out = self._out(x, row_idx) if out is None else out
+        return K.layernorm(x, self.weight, self.eps, out, deltas=self._deltas(delta), row_idx=row_idx)
+
+    def forward_pair(self, twin: "LayerNorm", x, delta=None):
+        if twin.width != self.width or twin.eps != self.eps or twin.weight.dtype != self.weight.dtype:
+            raise ValueError("two norms share a pass only with the same width, eps and weight type")
+        out, out2 = self._out(x, None), self._out(x, None)
+        K.layernorm(x, self.weight, self.eps, out, deltas=self._deltas(delta), weight2=twin.weight, out2=out2)
+        return out, out2

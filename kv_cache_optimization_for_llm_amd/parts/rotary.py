@@ -55,10 +55,45 @@ def llama3_frequencies(rot_dim: int, theta: float, *, factor: float, low_freq_fa
     return out.astype(f32)
 
 
+def plain_frequencies_f64(rot_dim: int, theta: float) -> np.ndarray:
+    """``theta^(-2i / rot)`` in float64: tables built from these hold the correctly rounded cos and
+    sin of ``position * frequency`` (an fp32 frequency times an fp32 position is off by up to
+    ``position * 6e-8`` radians)."""
+    i = np.arange(rot_dim // 2, dtype=np.float64)
+    return np.power(np.float64(theta), -2.0 * i / np.float64(rot_dim))
+
+
+def yarn_frequencies(rot_dim: int, theta: float, *, factor: float, original: float, fast: float,
+                     slow: float) -> np.ndarray:
+    """YaRN: pair i keeps its plain frequency ``f_i`` where it turns fast and takes ``f_i / factor``
+    where it turns slowly, blended linearly over the pair index between the pairs that make
+    ``fast`` and ``slow`` turns over ``original`` positions:
+    ``index(t) = rot ln(original / (2 pi t)) / (2 ln theta)``, ``lo = max(floor(index(fast)), 0)``,
+    ``hi = min(ceil(index(slow)), rot - 1)``, ``ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1)``,
+    ``f_i / factor * ramp_i + f_i * (1 - ramp_i)``.  float64.  (The rotation's magnitude,
+    ``0.1 ln(factor) + 1``, is the encoding's ``magnitude``: :func:`yarn_magnitude`.)"""
+    f = plain_frequencies_f64(rot_dim, theta)
+
+    def index(turns: float) -> float:
+        return rot_dim * math.log(float(original) / (2.0 * math.pi * float(turns))) / (2.0 * math.log(float(theta)))
+
+    lo = max(math.floor(index(fast)), 0)
+    hi = min(math.ceil(index(slow)), rot_dim - 1)
+    i = np.arange(rot_dim // 2, dtype=np.float64)
+    ramp = np.clip((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+    return f / float(factor) * ramp + f * (1.0 - ramp)
+
+
+def yarn_magnitude(factor: float) -> float:
+    return 0.1 * math.log(float(factor)) + 1.0
+
+
 # The rule that turns (rotary width, theta, parameters) into frequencies is chosen by name; another
 # scaling scheme is another entry here, registered from anywhere.
 ROTARY_FREQUENCIES.register("plain", plain_frequencies, replace=True)
 ROTARY_FREQUENCIES.register("llama3", llama3_frequencies, replace=True)
+ROTARY_FREQUENCIES.register("plain_f64", plain_frequencies_f64, replace=True)
+ROTARY_FREQUENCIES.register("yarn", yarn_frequencies, replace=True)
 
 
 def rotary_inv_freq(rot_dim: int, theta: float, scaling: Optional[dict]) -> np.ndarray:
@@ -72,13 +107,19 @@ def rotary_inv_freq(rot_dim: int, theta: float, scaling: Optional[dict]) -> np.n
 
 
 class _Tables:
-    """cos and sin of position * frequency, ``[positions, rot / 2]`` fp32 on one device."""
+    """cos and sin of position * frequency (times ``magnitude``), ``[positions, rot / 2]`` fp32 on
+    one device.  Angles are formed in the frequencies' own type: fp32 frequencies give the fp32
+    product, float64 frequencies the exact angle, rounded once at the end."""
 
-    def __init__(self, inv_freq: np.ndarray, positions: int, device):
-        pos = np.arange(positions, dtype=np.float32)[:, None]
-        angle = (pos * inv_freq[None, :]).astype(np.float32)
-        self.cos = torch.from_numpy(np.cos(angle).astype(np.float32)).to(device)
-        self.sin = torch.from_numpy(np.sin(angle).astype(np.float32)).to(device)
+    def __init__(self, inv_freq: np.ndarray, positions: int, device, magnitude: float = 1.0):
+        kind = inv_freq.dtype.type
+        pos = np.arange(positions, dtype=kind)[:, None]
+        angle = (pos * inv_freq[None, :]).astype(kind)
+        cos, sin = np.cos(angle), np.sin(angle)
+        if magnitude != 1.0:
+            cos, sin = cos * kind(magnitude), sin * kind(magnitude)
+        self.cos = torch.from_numpy(cos.astype(np.float32)).to(device)
+        self.sin = torch.from_numpy(sin.astype(np.float32)).to(device)
 
 
 # Tables are shared by every encoding with the same frequencies, length and device (the layers of
@@ -88,11 +129,11 @@ class _Tables:
 _TABLES: "weakref.WeakValueDictionary" = weakref.WeakValueDictionary()
 
 
-def shared_tables(inv_freq: np.ndarray, positions: int, device) -> _Tables:
-    key = (inv_freq.tobytes(), int(positions), str(torch.device(device)))
+def shared_tables(inv_freq: np.ndarray, positions: int, device, magnitude: float = 1.0) -> _Tables:
+    key = (inv_freq.tobytes(), str(inv_freq.dtype), float(magnitude), int(positions), str(torch.device(device)))
     hit = _TABLES.get(key)
     if hit is None:
-        hit = _TABLES[key] = _Tables(inv_freq, int(positions), device)
+        hit = _TABLES[key] = _Tables(inv_freq, int(positions), device, magnitude)
     return hit
 
 
@@ -101,15 +142,27 @@ class RotaryEncoding(PositionEncoding):
     graph_safe = True
 
     def __init__(self, *, head_dim: int, max_positions: int, theta: float, frequencies: str = "plain",
-                 frequency_params: Optional[dict] = None, rotary_dim: Optional[int] = None):
+                 frequency_params: Optional[dict] = None, rotary_dim: Optional[int] = None,
+                 pairing: str = "half", magnitude: float = 1.0, unit_norm_eps: Optional[float] = None):
+        """``pairing``: pair i of the rotated elements is (i, i + rot / 2) (``"half"``) or
+        (2i, 2i + 1) (``"interleaved"``).  ``magnitude`` multiplies cos and sin.  With
+        ``unit_norm_eps`` every query and key head is divided by its root mean square
+        (``sqrt(mean(x^2) + eps)``, over the whole head) after the rotation and before the key is
+        cached."""
         super().__init__("")
+        if pairing not in ("half", "interleaved"):
+            raise ValueError(f"rotary pairing {pairing!r} is not one of 'half', 'interleaved'")
+        self.pairing, self.magnitude = pairing, float(magnitude)
+        self.unit_norm_eps = None if unit_norm_eps is None else float(unit_norm_eps)
         self.head_dim = int(head_dim)
         self.rotary_dim = int(rotary_dim if rotary_dim is not None else head_dim)
         if self.rotary_dim % 2 or not 0 < self.rotary_dim <= self.head_dim:
             raise ValueError(f"rotary dim {self.rotary_dim} must be even and at most head_dim {head_dim}")
         self.max_positions = int(max_positions)
         self.inv_freq = np.asarray(ROTARY_FREQUENCIES.get(frequencies)(
-            self.rotary_dim, theta, **(frequency_params or {})), dtype=np.float32)
+            self.rotary_dim, theta, **(frequency_params or {})))
+        if self.inv_freq.dtype != np.float64:
+            self.inv_freq = self.inv_freq.astype(np.float32)
         if self.inv_freq.shape != (self.rotary_dim // 2,):
             raise ValueError(f"frequency rule {frequencies!r} gave {self.inv_freq.shape[0]} frequencies for a "
                              f"rotation over {self.rotary_dim} elements")
@@ -124,17 +177,25 @@ class RotaryEncoding(PositionEncoding):
 
     def tables(self, device) -> tuple:
         if self._tables is None or self._tables.cos.device != torch.device(device):
-            self._tables = shared_tables(self.inv_freq, self.max_positions, device)
+            self._tables = shared_tables(self.inv_freq, self.max_positions, device, self.magnitude)
         return self._tables.cos, self._tables.sin
 
     def rotate_half_tables(self, device, head_dim: int):
-        if self.rotary_dim != head_dim:
+        if self.rotary_dim != head_dim or self.pairing != "half" or self.unit_norm_eps is not None:
             return None
         return self.tables(device)
 
-    def apply_and_cache(self, qkv, positions, num_q_heads, num_kv_heads, head_dim, kv: Optional[KVView]):
+    def apply_and_cache(self, qkv, positions, num_q_heads, num_kv_heads, head_dim, kv: Optional[KVView],
+                        value_dim: Optional[int] = None):
         cos, sin = self.tables(qkv.device)
         write = kv is not None and kv.writes
+        value_dim = head_dim if value_dim is None else int(value_dim)
+        if self.pairing != "half" or self.unit_norm_eps is not None or value_dim != head_dim:
+            K.qk_encode_cache(qkv, positions, num_q_heads, num_kv_heads, head_dim, value_dim, cos, sin,
+                              self.pairing == "interleaved", self.unit_norm_eps,
+                              kv.k_cache if write else None, kv.v_cache if write else None,
+                              kv.slot_mapping if write else None)
+            return
         K.rope_kv_write(qkv, positions, num_q_heads, num_kv_heads, head_dim, cos, sin,
                         kv.k_cache if write else None, kv.v_cache if write else None,
                         kv.slot_mapping if write else None, kv.page_size if kv is not None else 0)
@@ -152,9 +213,14 @@ class NoPositionEncoding(PositionEncoding):
     def rotate_half_tables(self, device, head_dim: int):
         return (None, None)
 
-    def apply_and_cache(self, qkv, positions, num_q_heads, num_kv_heads, head_dim, kv: Optional[KVView]):
+    def apply_and_cache(self, qkv, positions, num_q_heads, num_kv_heads, head_dim, kv: Optional[KVView],
+                        value_dim: Optional[int] = None):
         write = kv is not None and kv.writes
         if not write:
+            return
+        if value_dim is not None and value_dim != head_dim:
+            K.qk_encode_cache(qkv, positions, num_q_heads, num_kv_heads, head_dim, value_dim, None, None, False,
+                              None, kv.k_cache, kv.v_cache, kv.slot_mapping)
             return
         K.rope_kv_write(qkv, positions, num_q_heads, num_kv_heads, head_dim, None, None,
                         kv.k_cache, kv.v_cache, kv.slot_mapping, kv.page_size)
