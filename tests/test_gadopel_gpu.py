@@ -1,0 +1,177 @@
+"""The Gadopel decoder in the engine against the plain implementation (``plain_gadopel``).
+
+Small configurations of their own (``gadopel_util``: other sizes, head counts, layer orders,
+windows and loops than any served model), seeded weights with spread-out attention and sinks of a
+few units.  Every schedule - whole prompts, token-by-token decoding, portions down to two tokens,
+mixed batches on a pool so small that pages and seats come back - must give the logits of the
+plain whole-sequence forward pass, in both number formats.
+"""
+import numpy as np
+import pytest
+import torch
+
+import gadopel_util as U
+import plain_gadopel as plain
+import replay_util as R
+from kv_cache_optimization_for_llm_amd.engine.engine import Engine, EngineOptions
+from kv_cache_optimization_for_llm_amd.engine.runner import LLM, ServeOptions
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    base = tmp_path_factory.mktemp("gadopel")
+    return {name: (cfg, *U.write_model(str(base / name), cfg, seed)) for name, (cfg, seed) in U.CONFIGS.items()}
+
+
+def engine_for(folder, dtype, **kw):
+    opts = dict(dtype=dtype, page_size=16, cache_tokens=1024, max_seqs=4, max_seq_len=512, max_batch_tokens=1024)
+    opts.update(kw)
+    return Engine(folder, EngineOptions(**opts))
+
+
+REQUESTS = {"P": [1, 2, 9, 40, 77], "Q": [3, 33, 70], "R": [1, 18, 50, 131]}
+
+
+def requests_for(name, cfg):
+    return {f"{name}{i}": U.prompt(cfg, n, 100 * i + n) for i, n in enumerate(REQUESTS[name])}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["P", "Q", "R"])
+def test_whole_prompts_and_the_first_tokens(name, dtype, models, gpu):
+    cfg, folder, state = models[name]
+    reqs = requests_for(name, cfg)
+    eng = engine_for(folder, dtype)
+    rows = U.run_steps(eng, R.whole(reqs))
+    assert len(rows) == sum(len(t) for t in reqs.values())
+    U.assert_rows(rows, U.expected_rows(cfg, state, reqs), dtype, "whole")
+    eng.cache.check()
+    assert eng.cache.free_seats == 4
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["P", "Q", "R"])
+def test_prefill_against_token_by_token_decoding(name, dtype, models, gpu):
+    """Most of a request in one step, the rest one token at a time: long enough that every window
+    passes over decoded tokens and leaves the kept first positions behind."""
+    cfg, folder, state = models[name]
+    reqs = {k: v for k, v in requests_for(name, cfg).items() if len(v) > 30}
+    eng = engine_for(folder, dtype)
+    rows = U.run_steps(eng, R.tail_decoded(reqs, tail=45))
+    U.assert_rows(rows, U.expected_rows(cfg, state, reqs), dtype, "decode")
+    # and a request decoded from its very first token on
+    first = {"solo": U.prompt(cfg, 60, 9)}
+    rows = U.run_steps(eng, R.tail_decoded(first, tail=59))
+    U.assert_rows(rows, U.expected_rows(cfg, state, first), dtype, "decode from the first token")
+    eng.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("sizes", [(2,), (7, 16, 5, 2, 33, 3, 64, 2), (17, 1, 1, 30)])
+@pytest.mark.parametrize("name", ["P", "R"])
+def test_portions_of_any_size(name, sizes, dtype, models, gpu):
+    cfg, folder, state = models[name]
+    reqs = {k: v for k, v in requests_for(name, cfg).items() if len(v) > 8}
+    eng = engine_for(folder, dtype, page_size=8 if name == "P" else 16)
+    rows = U.run_steps(eng, R.chunked(reqs, sizes))
+    U.assert_rows(rows, U.expected_rows(cfg, state, reqs), dtype, f"portions {sizes}")
+    eng.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name, seed", [("P", 0), ("Q", 1), ("R", 2), ("R", 3)])
+def test_mixed_batches_on_a_small_pool_reuse_pages_and_seats(name, seed, dtype, models, gpu):
+    cfg, folder, state = models[name]
+    lengths = [40, 3, 90, 25, 61, 2, 130, 47, 33]
+    reqs = {f"m{i}": U.prompt(cfg, n, 7 * i + seed) for i, n in enumerate(lengths)}
+    steps = R.mixed(reqs, seed=seed, max_live=3)
+    pool = R.max_live_tokens(steps, unit=16)
+    eng = engine_for(folder, dtype, cache_tokens=pool, max_seqs=3, max_seq_len=192)
+    rows = U.run_steps(eng, steps)
+    assert len(rows) == sum(lengths)
+    U.assert_rows(rows, U.expected_rows(cfg, state, reqs), dtype, "mixed")
+    eng.cache.check()
+    stats = eng.cache.stats()
+    assert stats["pages_reused"] > 0 and stats["running"] == 0
+    assert all(g.free_pages() == g.num_pages for g in eng.cache.groups)
+
+
+def test_a_request_alone_and_in_a_batch_give_the_same_32_bit_logits(models, gpu):
+    """fp32 logits of a (request, position) do not depend on the cut, the batch or the pages."""
+    cfg, folder, state = models["R"]
+    reqs = {f"b{i}": U.prompt(cfg, n, 50 + i) for i, n in enumerate([70, 21, 44])}
+    eng = engine_for(folder, "float32")
+    alone = U.run_steps(eng, R.whole(reqs))
+    together = U.run_steps(eng, R.mixed(reqs, seed=4, max_live=3, chunk_sizes=(2, 3, 16, 9)))
+    assert alone.keys() == together.keys()
+    for key in alone:
+        np.testing.assert_array_equal(alone[key], together[key], err_msg=str(key))
+
+
+def test_window_pages_are_given_back_and_the_kept_ones_stay(models, gpu):
+    cfg, folder, state = models["R"]
+    eng = engine_for(folder, "float32", cache_tokens=256)
+    toks = U.prompt(cfg, 200, 77)
+    reqs = {"w": toks}
+    rows = U.run_steps(eng, [{"step": 0, "entries": [{"id": "w", "tokens": toks[:150], "want": [149]}], "end": []}])
+    seat = eng.seat_of("w")
+    by_window = {g.spec.window: g for g in eng.cache.groups if g.spec.kind == "window"}
+    assert sorted(by_window) == [16, 33]
+    g = by_window[33]                       # 17 kept positions: blocks 0 and 1 stay; the window starts in block 7
+    row = g.table_host[seat]
+    assert (row[:2] >= 0).all() and (row[2:7] == -1).all() and (row[7:10] >= 0).all()
+    g = by_window[16]                       # 16 kept positions: block 0 stays
+    row = g.table_host[seat]
+    assert row[0] >= 0 and (row[1:8] == -1).all() and (row[8:10] >= 0).all()
+    more = U.run_steps(eng, [{"step": 1, "entries": [{"id": "w", "tokens": toks[150:], "want": [0, 49]}], "end": ["w"]}])
+    exp = U.expected_rows(cfg, state, reqs)
+    U.assert_rows(rows, exp, "float32")
+    got = {("w", 150 + p): v for (_, p), v in more.items()}
+    U.assert_rows(got, exp, "float32")
+    eng.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_trace_runner_replays_a_mixed_schedule(dtype, models, tmp_path, gpu):
+    cfg, folder, state = models["P"]
+    reqs = {f"t{i}": U.prompt(cfg, n, 11 + i) for i, n in enumerate([30, 2, 75, 18, 52])}
+    steps = R.mixed(reqs, seed=5, max_live=4)
+    rows = R.run_trace(folder, dtype, steps, R.max_live_tokens(steps), str(tmp_path / "out"), cfg["vocab"])
+    U.assert_rows(rows, U.expected_rows(cfg, state, reqs), dtype, "trace")
+    assert R.cache_stats(str(tmp_path / "out"))["pages_reused"] > 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["P", "R"])
+def test_greedy_generation_through_the_entry_point(name, dtype, models, gpu):
+    cfg, folder, state = models[name]
+    prompts = [U.prompt(cfg, n, 3 + n) for n in (1, 12, 37, 64, 5, 90)]
+    llm = LLM(folder, EngineOptions(dtype=dtype, max_seqs=3, max_seq_len=160, cache_tokens=480),
+              ServeOptions(chunk_size=16, max_batch_tokens=48))
+    got, reasons = llm.generate(prompts, max_new_tokens=24, ignore_eos=True, return_reasons=True)
+    assert reasons == ["length"] * len(prompts)
+    for p, g in zip(prompts, got):
+        assert len(g) == 24
+        logits = plain.forward(cfg, state, list(p) + list(g)).numpy()
+        for i, tok in enumerate(g):
+            row = logits[len(p) + i - 1]
+            slack = (1e-3 if dtype == "float32" else 6e-2) * (row.max() - row.mean())
+            assert row[tok] >= row.max() - slack, f"token {i}: {tok} is not the best ({int(row.argmax())})"
+    llm.engine.cache.check()
+    assert llm.engine.cache.free_seats == 3
+
+
+def test_decode_steps_from_graphs_equal_eager_steps(models, gpu):
+    """A bf16 decode step replayed from its HIP graph gives bit for bit what the eager step gives."""
+    cfg, folder, state = models["R"]
+    reqs = {f"g{i}": U.prompt(cfg, n, 31 + i) for i, n in enumerate([48, 80])}
+    steps = R.tail_decoded(reqs, tail=20)
+    eager = U.run_steps(engine_for(folder, "bfloat16", use_graphs=False), steps)
+    eng = engine_for(folder, "bfloat16")
+    assert eng.graphs is not None
+    replayed = U.run_steps(eng, steps)
+    assert eng.graphs.replays > 0
+    for key in eager:
+        np.testing.assert_array_equal(eager[key], replayed[key], err_msg=str(key))

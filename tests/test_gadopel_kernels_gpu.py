@@ -1,0 +1,251 @@
+"""The kernels behind the Gadopel parts, each alone against the plain functions of
+``plain_gadopel``: layer norm over a 32-bit stream, gated activations (own kernel and product
+epilogue), interleaved / partial / YaRN rotation with unit-norm heads and the cache write,
+attention with a window that keeps first positions, sinks and a value size of its own, and
+attention over low-rank rows.  Where random numbers would hide a fault - one far key among
+hundreds, a key just inside or just outside a window, at a page's edge - one query and one key
+are scaled so that this key's score stands out when (and only when) it is visible."""
+import numpy as np
+import pytest
+import torch
+
+import plain_gadopel as plain
+from kv_cache_optimization_for_llm_amd.ops import kernels as K
+from kv_cache_optimization_for_llm_amd.ops import latent_attention as lat_ops
+from kv_cache_optimization_for_llm_amd.parts.linear import Linear
+from kv_cache_optimization_for_llm_amd.parts.rotary import RotaryEncoding
+
+pytestmark = pytest.mark.gpu
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+TOL = {"float32": 2e-5, "bfloat16": 2e-2}
+
+
+def rnd(shape, seed, dtype=torch.float32, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+def close(got, want, tol, what=""):
+    got, want = got.double().cpu(), want.double().cpu()
+    err = (got - want).abs().max().item() / max(want.abs().max().item(), 1e-9)
+    assert err <= tol, f"{what}: off by {err:.3g} of the largest value (limit {tol})"
+
+
+@pytest.mark.parametrize("out_dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("width", [72, 96, 1000])
+def test_layer_norm_adds_pending_outputs_and_writes_two_copies(width, out_dtype, gpu):
+    x = rnd((7, width), 1, scale=3.0) + 1.5
+    d1, d2 = rnd((7, width), 2, DT[out_dtype]), rnd((7, width), 3, DT[out_dtype])
+    w1, w2 = (1 + 0.1 * rnd((width,), 4)).to(DT[out_dtype]), (1 + 0.1 * rnd((width,), 5)).to(DT[out_dtype])
+    xs = x.to(gpu)
+    o1 = torch.empty((7, width), dtype=DT[out_dtype], device=gpu)
+    o2 = torch.empty_like(o1)
+    K.layernorm(xs, w1.to(gpu), 1e-5, o1, deltas=(d1.to(gpu), d2.to(gpu)), weight2=w2.to(gpu), out2=o2)
+    total = x.double() + d1.double() + d2.double()
+    close(xs, total, 1e-6, "the stream after the add")          # the stream itself stays 32-bit
+    close(o1, plain.layer_norm(total, w1.double(), 1e-5), TOL[out_dtype], "first copy")
+    close(o2, plain.layer_norm(total, w2.double(), 1e-5), TOL[out_dtype], "second copy")
+    # gathered rows: nothing is written back, a row named twice is not added twice
+    idx = torch.tensor([6, 0, 6], dtype=torch.int32, device=gpu)
+    before = xs.clone()
+    o3 = torch.empty((3, width), dtype=DT[out_dtype], device=gpu)
+    K.layernorm(xs, w1.to(gpu), 1e-5, o3, deltas=(d1.to(gpu),), row_idx=idx)
+    assert torch.equal(xs, before)
+    tol = TOL[out_dtype]
+    close(o3, plain.layer_norm((total + d1.double())[[6, 0, 6]], w1.double(), 1e-5), tol, "gathered rows")
+
+
+@pytest.mark.parametrize("activation", ["relu", "gelu_tanh", "silu"])
+@pytest.mark.parametrize("rows", [1, 2, 8, 40, 200])
+def test_gated_activations_alone_and_in_the_product(rows, activation, gpu):
+    act = {"relu": torch.relu, "silu": torch.nn.functional.silu,
+           "gelu_tanh": lambda z: 0.5 * z * (1 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))}[activation]
+    inter, width = 96, 64
+    x = rnd((rows, width), 1, torch.bfloat16)
+    w = rnd((2 * inter, width), 2, torch.bfloat16, 0.3)
+    gu = x.double() @ w.double().T
+    want = act(gu[:, :inter]) * gu[:, inter:]
+    for dtype in ("float32", "bfloat16"):
+        out = torch.empty((rows, inter), dtype=DT[dtype], device=gpu)
+        K.act_mul(gu.to(DT[dtype]).to(gpu), out, activation)
+        close(out, want, TOL[dtype], f"act_mul {dtype}")
+    lin = Linear(w.to(gpu), halves=2)
+    if lin.fused_kernel(rows, torch.bfloat16) is not None:
+        out = torch.empty((rows, inter), dtype=torch.bfloat16, device=gpu)
+        lin.gated(x.to(gpu), out, activation)
+        close(out, want, 2e-2, "the product's epilogue")
+
+
+def cache_for(length, page_size, seed):
+    """A block table that scatters the positions' pages, and the slots of positions 0..length-1."""
+    blocks = (length + page_size - 1) // page_size
+    perm = np.random.default_rng(seed).permutation(blocks + 3)[:blocks]
+    table = torch.full((2, blocks + 2), -1, dtype=torch.int32)
+    table[1, :blocks] = torch.from_numpy(perm.astype(np.int32))
+    pos = np.arange(length)
+    slots = torch.from_numpy((perm[pos // page_size] * page_size + pos % page_size).astype(np.int32))
+    return table, slots, blocks + 3
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("heads, kv_heads, dim, vdim, rot, interleaved, unit", [
+    (4, 2, 32, 16, 16, True, True), (3, 3, 20, 20, 12, True, True), (2, 1, 64, 64, 64, True, False),
+    (6, 2, 48, 24, 32, False, True), (2, 2, 16, 40, 0, True, True)])
+def test_rotation_unit_norm_and_cache_write(heads, kv_heads, dim, vdim, rot, interleaved, unit, dtype, gpu):
+    T, page = 37, 8
+    eps = 1e-5
+    scaling = {"factor": 8.0, "original": 48, "fast": 6.0, "slow": 1.5}
+    table, slots, pages = cache_for(T, page, 3)
+    qkv = rnd((T, heads * dim + kv_heads * dim + kv_heads * vdim), 7, DT[dtype])
+    positions = torch.arange(100, 100 + T, dtype=torch.int32)
+    cos = sin = None
+    if rot:
+        enc = RotaryEncoding(head_dim=dim, rotary_dim=rot, max_positions=256, theta=777.0, frequencies="yarn",
+                             frequency_params=scaling, magnitude=0.1 * np.log(8.0) + 1,
+                             pairing="interleaved" if interleaved else "half")
+        cos, sin = enc.tables(gpu)
+    k_cache = torch.zeros((pages, *K.k_page_shape(kv_heads, dim)[:2], page, K.k_chunk(dim)), dtype=DT[dtype], device=gpu)
+    v_cache = torch.zeros((pages, kv_heads, vdim, page), dtype=DT[dtype], device=gpu)
+    dev = qkv.to(gpu)
+    K.qk_encode_cache(dev, positions.to(gpu), heads, kv_heads, dim, vdim, cos, sin, interleaved,
+                      eps if unit else None, k_cache, v_cache, slots.to(gpu))
+    src = qkv.double()
+    q = src[:, :heads * dim].view(T, heads, dim)
+    k = src[:, heads * dim:(heads + kv_heads) * dim].view(T, kv_heads, dim)
+    v = src[:, (heads + kv_heads) * dim:].view(T, kv_heads, vdim)
+    if rot:
+        freqs, mag = plain.rotary_frequencies(rot, 777.0, scaling)
+        q = plain.rotate(q, positions, freqs, mag, interleaved)
+        k = plain.rotate(k, positions, freqs, mag, interleaved)
+    if unit:
+        q, k = plain.unit_rms(q, eps), plain.unit_rms(k, eps)
+    close(dev[:, :heads * dim].view(T, heads, dim), q, TOL[dtype], "queries")
+    got_k = K.pages_to_keys(k_cache).reshape(pages, kv_heads, page, dim)
+    sl = slots.long()
+    close(got_k[sl // page, :, sl % page], k, TOL[dtype], "cached keys")
+    close(v_cache[sl // page, :, :, sl % page], v, 1e-9, "cached values")
+
+
+def standout(q, k, query_pos, key_pos, head, kv_head, strength=12.0):
+    """Makes key ``key_pos`` the one query ``query_pos`` of ``head`` scores highest by far."""
+    direction = q[query_pos, head] / q[query_pos, head].norm()
+    k[key_pos, kv_head] = direction * strength
+    q[query_pos, head] = direction * strength
+
+
+CASES = [  # (length, window, keep_first, query position, key that stands out)
+    (300, 0, 0, 299, 0), (300, 0, 0, 299, 157),                     # far keys, no window
+    (300, 40, 20, 299, 260), (300, 40, 20, 299, 259),              # just inside / outside the window
+    (300, 40, 20, 299, 19), (300, 40, 20, 299, 20),                # the last kept position / the first that is not
+    (300, 40, 20, 45, 20), (300, 40, 20, 59, 20), (300, 40, 20, 60, 20),
+    (130, 16, 16, 129, 15), (130, 16, 16, 129, 16), (130, 16, 16, 129, 113), (130, 16, 16, 129, 114),   # page edges
+    (70, 64, 0, 69, 5), (70, 64, 0, 69, 6), (5, 3, 1, 4, 0), (5, 3, 1, 4, 1), (1, 0, 0, 0, 0),
+]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("length, window, keep_first, qpos, kpos", CASES)
+def test_attention_sees_exactly_the_visible_keys(length, window, keep_first, qpos, kpos, dtype, gpu):
+    heads, kv_heads, dim, vdim, page, scale = 4, 2, 24, 40, 16, 0.3
+    q, k, v = rnd((length, heads, dim), 1), rnd((length, kv_heads, dim), 2), rnd((length, kv_heads, vdim), 3)
+    standout(q, k, qpos, kpos, head=2, kv_head=1)
+    v[kpos, 1] = 5.0
+    q, k, v = (t.to(DT[dtype]) for t in (q, k, v))
+    sinks = torch.tensor([0.5, -1.0, 2.0, 0.0])
+    table, slots, pages = cache_for(length, page, 11)
+    k_cache = torch.zeros((pages, *K.k_page_shape(kv_heads, dim)[:2], page, K.k_chunk(dim)), dtype=DT[dtype], device=gpu)
+    v_cache = torch.full((pages, kv_heads, vdim, page), float("nan"), dtype=DT[dtype], device=gpu)      # pages of others
+    sl = slots.long()
+    kp = K.pages_to_keys(k_cache).reshape(pages, kv_heads, page, dim)
+    kp[sl // page, :, sl % page] = k.to(gpu)
+    k_cache.copy_(K.keys_to_pages(kp))
+    v_cache[sl // page, :, :, sl % page] = v.to(gpu)
+    rows = sorted({qpos, 0, length - 1, min(length - 1, max(0, keep_first)), length // 2})
+    tok_pos = torch.tensor(rows, dtype=torch.int32)
+    out = torch.empty((len(rows), heads * vdim), dtype=DT[dtype], device=gpu)
+    K.attention_rowwise(q[rows].reshape(len(rows), -1).contiguous().to(gpu), heads * dim, out, k_cache, v_cache,
+                        table.to(gpu), torch.ones(len(rows), dtype=torch.int32, device=gpu), tok_pos.to(gpu),
+                        heads, kv_heads, dim, scale, window, keep_first, sinks.to(gpu), vdim)
+    qd, kd, vd = q.double(), k.double().repeat_interleave(2, dim=1), v.double().repeat_interleave(2, dim=1)
+    prob = plain.softmax_rows(torch.einsum("ihd,jhd->hij", qd, kd) * scale, plain.visible(length, window, keep_first),
+                              sinks.double())
+    want = torch.einsum("hij,jhd->ihd", prob, vd)[rows].reshape(len(rows), -1)
+    assert torch.isfinite(out).all()
+    close(out, want, TOL[dtype] * 5, "attention")
+    seen = plain.visible(length, window, keep_first)[qpos, kpos].item()
+    got = out.view(len(rows), heads, vdim)[rows.index(qpos), 2].float().mean().item()
+    assert (got > 2.5) == bool(seen), f"the key that stands out is {'visible' if seen else 'hidden'}, the output says {got:.2f}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("length, window, keep_first, qpos, kpos", CASES)
+def test_latent_attention_sees_exactly_the_visible_rows(length, window, keep_first, qpos, kpos, dtype, gpu):
+    heads, rank, rot, page, scale = 3, 40, 8, 16, 0.25
+    kd = rank + rot
+    q, rows_kv = rnd((length, heads, kd), 4), rnd((length, 1, kd), 5)
+    standout(q, rows_kv, qpos, kpos, head=1, kv_head=0, strength=14.0)
+    q, rows_kv = q.to(DT[dtype]), rows_kv.to(DT[dtype])
+    sinks = torch.tensor([1.0, -2.0, 0.3])
+    table, slots, pages = cache_for(length, page, 13)
+    cache = torch.full((pages, page, kd), float("nan"), dtype=DT[dtype], device=gpu)
+    cache.view(-1, kd)[slots.long()] = rows_kv[:, 0].to(gpu)
+    picks = sorted({qpos, 0, length - 1, length // 2})
+
+    class Batch:
+        tok_seat = torch.ones(len(picks), dtype=torch.int32, device=gpu)
+        positions = torch.tensor(picks, dtype=torch.int32, device=gpu)
+
+    class View:
+        arrays = {"latent": cache}
+        block_table = table.to(gpu)
+        page_size = page
+
+    out = torch.empty((len(picks), heads, rank), dtype=DT[dtype], device=gpu)
+    lat_ops.latent_attention(q[picks].contiguous().to(gpu), out, View, Batch, scale, window, keep_first, sinks.to(gpu))
+    qd, kdbl = q.double(), rows_kv.double().expand(length, heads, kd)
+    prob = plain.softmax_rows(torch.einsum("ihd,jhd->hij", qd, kdbl) * scale, plain.visible(length, window, keep_first),
+                              sinks.double())
+    want = torch.einsum("hij,jd->ihd", prob, rows_kv.double()[:, 0, :rank])[picks]
+    assert torch.isfinite(out).all()
+    close(out, want, TOL[dtype] * 5, "latent attention")
+    seen = plain.visible(length, window, keep_first)[qpos, kpos].item()
+    weight = (out[picks.index(qpos), 1].double().cpu() @ rows_kv.double()[kpos, 0, :rank]) / rows_kv.double()[kpos, 0, :rank].norm() ** 2
+    assert (weight.item() > 0.5) == bool(seen)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_low_rank_entry_is_normed_rotated_and_cached(dtype, gpu):
+    T, heads, dim, rot, rank, page, eps = 21, 3, 16, 8, 40, 8, 1e-5
+    kd = rank + rot
+    y = rnd((T, heads * (dim + rot) + kd + heads), 3, DT[dtype])
+    w = (1 + 0.2 * rnd((rank,), 4)).to(DT[dtype])
+    positions = torch.arange(50, 50 + T, dtype=torch.int32)
+    table, slots, pages = cache_for(T, page, 5)
+    enc = RotaryEncoding(head_dim=rot, max_positions=128, theta=300.0, frequencies="plain_f64")
+    cos, sin = enc.tables(gpu)
+    cache = torch.zeros((pages, page, kd), dtype=DT[dtype], device=gpu)
+    q_lat = torch.zeros((T, heads, kd), dtype=DT[dtype], device=gpu)
+    K.latent_encode_cache(y.to(gpu), heads * (dim + rot), q_lat, cache, w.to(gpu), eps, cos, sin, positions.to(gpu),
+                          slots.to(gpu), heads, dim, rank)
+    freqs, mag = plain.rotary_frequencies(rot, 300.0)
+    yd = y.double()
+    q_rot = plain.rotate(yd[:, :heads * (dim + rot)].view(T, heads, dim + rot)[..., dim:], positions, freqs, mag, False)
+    entry = yd[:, heads * (dim + rot):heads * (dim + rot) + kd]
+    c = plain.unit_rms(entry[:, :rank], eps) * w.double()
+    k_rot = plain.rotate(entry[:, rank:], positions, freqs, mag, False)
+    close(q_lat[:, :, rank:], q_rot, TOL[dtype], "rotated query parts")
+    got = cache.view(-1, kd)[slots.long().to(gpu)]
+    close(got[:, :rank], c, TOL[dtype], "latent")
+    close(got[:, rank:], k_rot, TOL[dtype], "rotated key part")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("rows, heads, n, k", [(1, 3, 40, 16), (9, 5, 24, 8), (130, 2, 70, 96), (3, 1, 8, 200)])
+def test_per_head_products_into_column_ranges(rows, heads, n, k, dtype, gpu):
+    x_wide = rnd((rows, heads, k + 5), 1, DT[dtype]).to(gpu)
+    out_wide = torch.zeros((rows, heads, n + 3), dtype=DT[dtype], device=gpu)
+    w = rnd((heads, n, k), 2, DT[dtype], 0.3).to(gpu)
+    lat_ops.heads_product(x_wide[:, :, :k], w, out_wide[:, :, :n])
+    want = torch.einsum("thk,hnk->thn", x_wide[:, :, :k].double(), w.double())
+    close(out_wide[:, :, :n], want, TOL[dtype], "per-head product")
+    assert (out_wide[:, :, n:] == 0).all()
