@@ -145,7 +145,8 @@ __device__ inline void rotate_pair(const T *src, T *dst, int i, int rot, int int
 template <typename T, typename TW>
 __global__ void __launch_bounds__(256)
 latent_encode_cache_kernel(const T *__restrict__ y, int row_stride, int kv_off, T *__restrict__ q_lat,
-                           T *__restrict__ cache, const TW *__restrict__ norm_weight, float eps,
+                           T *__restrict__ cache, T *__restrict__ cache_t, int page_size,
+                           const TW *__restrict__ norm_weight, float eps,
                            const float *__restrict__ cos_table, const float *__restrict__ sin_table,
                            const int *__restrict__ positions, const int *__restrict__ slot_mapping, int heads,
                            int plain_dim, int rank, int rot, int interleaved) {
@@ -170,13 +171,18 @@ latent_encode_cache_kernel(const T *__restrict__ y, int row_stride, int kv_off, 
         sq += v * v;
     }
     const float inv = 1.0f / sqrtf(block_sum(sq, red_s, blockDim.x / KVA_WAVE) / (float)rank + eps);
-    for (int j = threadIdx.x; j < rank; j += blockDim.x)
-        dst[j] = from_float<T>(to_float(c[j]) * inv * to_float(norm_weight[j]));
+    // (the latent a second time, transposed inside its page [rank, page_size], where a kernel reads it that way)
+    T *dst_t = cache_t ? cache_t + (size_t)(slot / page_size) * rank * page_size + slot % page_size : nullptr;
+    for (int j = threadIdx.x; j < rank; j += blockDim.x) {
+        const T v = from_float<T>(to_float(c[j]) * inv * to_float(norm_weight[j]));
+        dst[j] = v;
+        if (dst_t) dst_t[(size_t)j * page_size] = v;
+    }
     for (int i = threadIdx.x; i < half; i += blockDim.x) rotate_pair(c + rank, dst + rank, i, rot, interleaved, cs, sn);
 }
 
 extern "C" int kva_latent_encode_cache(const void *y, int row_stride, int kv_off, void *q_lat, void *cache,
-                                       const void *norm_weight, int weight_dtype, float eps, const float *cos_table,
+                                       void *cache_t, int page_size, const void *norm_weight, int weight_dtype, float eps, const float *cos_table,
                                        const float *sin_table, const int *positions, const int *slot_mapping,
                                        int tokens, int heads, int plain_dim, int rank, int rot, int interleaved,
                                        int dtype, hipStream_t stream) {
@@ -186,11 +192,13 @@ extern "C" int kva_latent_encode_cache(const void *y, int row_stride, int kv_off
     KVA_REQUIRE(kv_off >= heads * (plain_dim + rot) && row_stride >= kv_off + rank + rot,
                 "latent_encode_cache: the row layout [queries | entry] does not fit its stride");
     KVA_REQUIRE(!slot_mapping || cache, "latent_encode_cache: cache write asked for without a cache");
+    KVA_REQUIRE(!cache_t || page_size > 0, "latent_encode_cache: the transposed copy needs the page size");
     KVA_REQUIRE(dtype == KVA_F32 || dtype == KVA_BF16, "latent_encode_cache: unsupported dtype %d", dtype);
     if (tokens == 0) return KVA_OK;
 #define LAUNCH_LE(T, TW)                                                                                        \
     hipLaunchKernelGGL((latent_encode_cache_kernel<T, TW>), dim3(tokens), dim3(256), 0, stream, (const T *)y,   \
-                       row_stride, kv_off, (T *)q_lat, (T *)cache, (const TW *)norm_weight, eps, cos_table,      \
+                       row_stride, kv_off, (T *)q_lat, (T *)cache, (T *)cache_t, page_size,                     \
+                       (const TW *)norm_weight, eps, cos_table,                                                 \
                        sin_table, positions, slot_mapping, heads, plain_dim, rank, rot, interleaved)
     if (dtype == KVA_F32 && weight_dtype == KVA_F32) LAUNCH_LE(float, float);
     else if (dtype == KVA_BF16 && weight_dtype == KVA_BF16) LAUNCH_LE(bf16_t, bf16_t);

@@ -419,6 +419,54 @@ def latent_attention_rowwise(q: torch.Tensor, out: torch.Tensor, cache: torch.Te
     return out
 
 
+def latent_attention_mfma_supported(rank: int, key_dim: int, page_size: int) -> bool:
+    return bool(hip_lib().kva_latent_attention_mfma_supported(int(rank), int(key_dim), int(page_size)))
+
+
+def latent_attention_mfma(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, cache_t: torch.Tensor,
+                          block_table: torch.Tensor, item_entry: torch.Tensor, item_row0: torch.Tensor,
+                          entry_seat: torch.Tensor, entry_q_start: torch.Tensor, entry_start_pos: torch.Tensor,
+                          scale: float, window: int = 0, keep_first: int = 0, sinks: Optional[torch.Tensor] = None,
+                          splits: int = 1, per_split: int = 0) -> torch.Tensor:
+    """:func:`latent_attention_rowwise` on the matrix cores (bf16): ``cache_t`` ``[pages, rank,
+    page_size]`` is the latent part of the rows once more, transposed; a work item is 16 rows
+    ``token_in_entry * heads + head`` of entry ``item_entry[i]`` from ``item_row0[i]`` on.  With
+    ``splits`` > 1 the keys are cut into ranges of ``per_split`` (a multiple of 32), one wavefront
+    each, and a second kernel adds their results up."""
+    if q.dim() != 3 or out.dim() != 3 or cache.dim() != 3 or cache_t.dim() != 3 or q.shape[:2] != out.shape[:2]:
+        raise KernelError("latent_attention_mfma: q [T, heads, key_dim], out [T, heads, rank], cache [pages, page, key_dim]")
+    tokens, heads, key_dim = q.shape
+    rank, pages, page_size = out.shape[2], cache.shape[0], cache.shape[1]
+    if cache.shape[2] != key_dim or tuple(cache_t.shape) != (pages, rank, page_size):
+        raise KernelError(f"latent_attention_mfma: cache {tuple(cache.shape)} / transposed {tuple(cache_t.shape)} do not fit "
+                          f"rows of {key_dim} with rank {rank}")
+    if not (q.dtype == out.dtype == cache.dtype == cache_t.dtype == torch.bfloat16):
+        raise KernelError("latent_attention_mfma: bfloat16 only")
+    if not latent_attention_mfma_supported(rank, key_dim, page_size):
+        raise KernelError(f"latent_attention_mfma: no instance for rank {rank}, rows of {key_dim}, pages of {page_size}")
+    n = item_entry.shape[0]
+    entries = entry_seat.shape[0]
+    if item_row0.shape != (n,) or entry_q_start.shape != (entries + 1,) or entry_start_pos.shape != (entries,):
+        raise KernelError("latent_attention_mfma: one row0 per item, entries + 1 starts, one start position per entry")
+    if sinks is not None and (sinks.shape != (heads,) or sinks.dtype != torch.float32):
+        raise KernelError("latent_attention_mfma: sinks are fp32, one per head")
+    part_o = part_ml = None
+    if splits > 1:
+        if per_split <= 0 or per_split % 32:
+            raise KernelError("latent_attention_mfma: key ranges are multiples of 32 keys")
+        part_o = torch.empty((tokens * heads, splits, rank), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((tokens * heads, splits, 2), dtype=torch.float32, device=q.device)
+    check(hip_lib().kva_latent_attention_mfma(
+        _dev(out, "out"), _opt(part_o, "part_o"), _opt(part_ml, "part_ml"), _dev(q, "q"), _dev(cache, "cache"),
+        _dev(cache_t, "cache_t"), _dev(block_table, "block_table", torch.int32), block_table.shape[1],
+        _dev(item_entry, "item_entry", torch.int32), _dev(item_row0, "item_row0", torch.int32),
+        _dev(entry_seat, "entry_seat", torch.int32), _dev(entry_q_start, "entry_q_start", torch.int32),
+        _dev(entry_start_pos, "entry_start_pos", torch.int32), n, tokens * heads, heads, rank, key_dim, page_size,
+        float(scale), int(window), int(keep_first), _opt(sinks, "sinks"), int(splits), int(per_split), _stream()),
+        "latent_attention_mfma")
+    return out
+
+
 def layernorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor, deltas=(),
               row_idx: Optional[torch.Tensor] = None, weight2: Optional[torch.Tensor] = None,
               out2: Optional[torch.Tensor] = None, rms: bool = False) -> torch.Tensor:
@@ -533,11 +581,12 @@ def qk_encode_cache(qkv: torch.Tensor, positions: torch.Tensor, num_q_heads: int
 def latent_encode_cache(y: torch.Tensor, kv_off: int, q_lat: torch.Tensor, cache: Optional[torch.Tensor],
                         norm_weight: torch.Tensor, eps: float, cos: torch.Tensor, sin: torch.Tensor,
                         positions: torch.Tensor, slot_mapping: Optional[torch.Tensor], heads: int, plain_dim: int,
-                        rank: int, interleaved: bool = False) -> None:
+                        rank: int, interleaved: bool = False, cache_t: Optional[torch.Tensor] = None) -> None:
     """From a projection row ``y[t] = [heads x (plain_dim + rot) | ... rank + rot at kv_off ...]``:
     the rotated part of every query head goes to ``q_lat[t, h, rank:]``; the entry's first ``rank``
     elements, RMS-normed with ``norm_weight``, and its rotated last ``rot`` go to row
-    ``slot_mapping[t]`` of ``cache`` ``[pages, page_size, rank + rot]``."""
+    ``slot_mapping[t]`` of ``cache`` ``[pages, page_size, rank + rot]`` - and the normed latent a
+    second time into ``cache_t`` ``[pages, rank, page_size]`` where that is given."""
     tokens = y.shape[0]
     rot = 2 * cos.shape[1]
     if y.dim() != 2 or q_lat.shape != (tokens, heads, rank + rot) or q_lat.dtype != y.dtype or positions.shape != (tokens,):
@@ -548,8 +597,11 @@ def latent_encode_cache(y: torch.Tensor, kv_off: int, q_lat: torch.Tensor, cache
     if write and (cache.dim() != 3 or cache.shape[2] != rank + rot or cache.dtype != y.dtype
                   or slot_mapping.shape != (tokens,)):
         raise KernelError("latent_encode_cache: cache [pages, page_size, rank + rot] of y's dtype, one slot per token")
+    if cache_t is not None and write and (cache_t.shape != (cache.shape[0], rank, cache.shape[1]) or cache_t.dtype != y.dtype):
+        raise KernelError("latent_encode_cache: the transposed copy must be [pages, rank, page_size] of y's dtype")
     check(hip_lib().kva_latent_encode_cache(
         _dev(y, "y"), y.shape[1], int(kv_off), _dev(q_lat, "q_lat"), _opt(cache if write else None, "cache"),
+        _opt(cache_t if write else None, "cache_t"), cache.shape[1] if write else 0,
         _dev(norm_weight, "norm_weight"), dtype_code(norm_weight.dtype), float(eps),
         _dev(cos, "cos", torch.float32), _dev(sin, "sin", torch.float32), _dev(positions, "positions", torch.int32),
         _opt(slot_mapping if write else None, "slot_mapping", torch.int32), tokens, heads, plain_dim, rank, rot,

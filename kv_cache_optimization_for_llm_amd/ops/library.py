@@ -50,7 +50,9 @@ _HIP_SIGNATURES = {
     "kva_act_mul": [P, P, I, I, I, I, P],
     "kva_head_gate": [P, P, I, I, I, I, I, P],
     "kva_qk_encode_cache": [P, I, I, I, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P],
-    "kva_latent_encode_cache": [P, I, I, P, P, P, I, F, P, P, P, P, I, I, I, I, I, I, I, P],
+    "kva_latent_encode_cache": [P, I, I, P, P, P, I, P, I, F, P, P, P, P, I, I, I, I, I, I, I, P],
+    "kva_latent_attention_mfma_supported": [I, I, I],
+    "kva_latent_attention_mfma": [P, P, P, P, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P, I, I, P],
     "kva_heads_matmul": [P, I, I, P, I, I, P, I, I, I, I, I, P],
     "kva_attention_mfma": [P, P, P, P, I, P, P, P, I, P, P, P, I, I, P, P, P, I, I, I, I, I, F, I, I, I, I, I, I, I, P],
     "kva_attention_mfma_rope": [P, P, P, P, I, P, P, P, I, P, I, I, I, I, I, I, F, I, I, I, I, P, P, P, I, P],

@@ -35,10 +35,15 @@ from .base import CacheArray, KVCacheSpec, Mixer, MixerContext, NormedRows
 from .linear import Linear
 
 
-def latent_cache_spec(rank: int, rot_dim: int, kind: str = "full", window: int = 0, keep_first: int = 0) -> KVCacheSpec:
-    """One row ``[latent (rank) ; rotated key part (rot_dim)]`` per token, pages ``[page_size, rank + rot_dim]``."""
-    return KVCacheSpec((CacheArray("latent", (int(rank) + int(rot_dim),), token_axis=0),), kind, int(window),
-                       int(keep_first) if kind == "window" else 0)
+def latent_cache_spec(rank: int, rot_dim: int, kind: str = "full", window: int = 0, keep_first: int = 0,
+                      transposed: bool = False) -> KVCacheSpec:
+    """One row ``[latent (rank) ; rotated key part (rot_dim)]`` per token, pages ``[page_size, rank +
+    rot_dim]``; with ``transposed`` the latent a second time in pages ``[rank, page_size]``, the
+    layout in which the matrix-core kernel reads it as the values' operand."""
+    arrays = (CacheArray("latent", (int(rank) + int(rot_dim),), token_axis=0),)
+    if transposed:
+        arrays += (CacheArray(lat_ops.TRANSPOSED, (int(rank),), token_axis=1),)
+    return KVCacheSpec(arrays, kind, int(window), int(keep_first) if kind == "window" else 0)
 
 
 @MIXERS.register("latent_attention")
@@ -104,8 +109,12 @@ class LatentAttention(Mixer):
         self.sinks = tensors[n["sink"]].to(torch.float32).contiguous() if self.has_sink else None
 
     def kv_cache_spec(self) -> KVCacheSpec:
+        # a bf16 model at sizes the matrix-core kernel has an instance for keeps the transposed copy
+        # it reads (asked after load(): the weights' type is the compute type)
+        fast = self.proj is not None and self.proj.weight.dtype == torch.bfloat16 and self.proj.weight.is_cuda \
+            and lat_ops.mfma_supported(self.rank, self.key_dim)
         return latent_cache_spec(self.rank, self.rot_dim, kind="window" if self.window > 0 else "full",
-                                 window=self.window, keep_first=self.keep_first)
+                                 window=self.window, keep_first=self.keep_first, transposed=fast)
 
     def activation_elements(self) -> int:
         H = self.num_heads
@@ -125,7 +134,8 @@ class LatentAttention(Mixer):
         write = kv.writes
         K.latent_encode_cache(y, self.kv_off, q_lat, kv.arrays["latent"] if write else None, self.norm_weight,
                               self.norm_eps, cos, sin, batch.positions, kv.slot_mapping if write else None, H,
-                              self.head_dim, self.rank, interleaved=self.position.pairing == "interleaved")
+                              self.head_dim, self.rank, interleaved=self.position.pairing == "interleaved",
+                              cache_t=kv.arrays.get(lat_ops.TRANSPOSED) if write else None)
         # the key expansion on the query side: q_lat[:, h, :rank] = U_k[h]^T q_p[h]
         q_plain = y[:, :self.kv_off].view(T, H, self.head_dim + self.rot_dim)[:, :, :self.head_dim]
         lat_ops.heads_product(q_plain, self.up_k_t, q_lat[:, :, :self.rank])

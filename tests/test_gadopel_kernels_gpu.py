@@ -249,3 +249,45 @@ def test_per_head_products_into_column_ranges(rows, heads, n, k, dtype, gpu):
     want = torch.einsum("thk,hnk->thn", x_wide[:, :, :k].double(), w.double())
     close(out_wide[:, :, :n], want, TOL[dtype], "per-head product")
     assert (out_wide[:, :, n:] == 0).all()
+
+
+@pytest.mark.parametrize("per_range", [0, 32, 96])
+@pytest.mark.parametrize("heads, rank, rot, window, keep_first", [
+    (3, 64, 32, 0, 0), (16, 64, 64, 0, 0), (5, 128, 32, 40, 20), (20, 64, 32, 33, 0), (6, 128, 64, 16, 16)])
+def test_latent_attention_on_the_matrix_cores(heads, rank, rot, window, keep_first, per_range, gpu):
+    """Entries of a step - two portions of prompts cut in the middle of pages and of tiles, and
+    decoded tokens, one right behind a page's edge - against the plain attention over all rows;
+    the keys whole and in ranges.  Pages of other requests, and the rest of a request's last page,
+    hold NaN."""
+    page, scale, length = 16, 0.2, 200
+    kd = rank + rot
+    assert K.latent_attention_mfma_supported(rank, kd, page)
+    q_all = rnd((length, heads, kd), 21, torch.bfloat16)
+    rows_kv = rnd((length, kd), 22, torch.bfloat16)
+    sinks = rnd((heads,), 23) * 2
+    table, slots, pages = cache_for(length, page, 17)
+    entries = [(37, 30), (199, 1), (0, 9), (112, 1), (96, 16)]        # (first position, tokens) of one request's copies
+    lat = torch.full((pages, page, kd), float("nan"), dtype=torch.bfloat16, device=gpu)
+    lat_t = torch.full((pages, rank, page), float("nan"), dtype=torch.bfloat16, device=gpu)
+    prob = plain.softmax_rows(torch.einsum("ihd,jd->hij", q_all.double(), rows_kv.double()) * scale,
+                              plain.visible(length, window, keep_first), sinks.double())
+    want_all = torch.einsum("hij,jd->ihd", prob, rows_kv.double()[:, :rank])
+    for start, n in entries:
+        # what the request holds when this entry runs: positions up to its last token
+        upto = start + n
+        lat.fill_(float("nan")); lat_t.fill_(float("nan"))
+        sl = slots[:upto].long().to(gpu)
+        lat.view(-1, kd)[sl] = rows_kv[:upto].to(gpu)
+        tmp = lat_t.permute(0, 2, 1).reshape(-1, rank)                  # (a copy: written back below)
+        tmp[sl] = rows_kv[:upto, :rank].to(gpu)
+        lat_t.copy_(tmp.view(pages, page, rank).permute(0, 2, 1))
+        q = q_all[start:upto].contiguous().to(gpu)
+        tiles = (n * heads + 15) // 16
+        out = torch.empty((n, heads, rank), dtype=torch.bfloat16, device=gpu)
+        ranges = 1 if per_range == 0 else -(-upto // per_range)
+        i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=gpu)
+        K.latent_attention_mfma(q, out, lat, lat_t, table.to(gpu), i32([0] * tiles), i32([16 * t for t in range(tiles)]),
+                                i32([1]), i32([0, n]), i32([start]), scale, window, keep_first, sinks.to(gpu),
+                                ranges, per_range)
+        assert torch.isfinite(out.float()).all(), f"entry {start}+{n}"
+        close(out, want_all[start:upto], 3e-2, f"entry {start}+{n}")
