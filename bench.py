@@ -14,6 +14,13 @@ tokens, each with its step time, bytes and fraction of the HBM peak, and the ser
 ``points`` also holds the device time per class of kernel of one decode step and of the prefill
 (``kclass_...``; ``--no-kernel-classes`` leaves them out) and, for the serving runs, pages reused,
 preemptions and fragmentation failures.
+
+    python bench.py --design gadopel [--layers 8]
+
+is another measurement with a JSON line of its own (the default run above is untouched): prefill
+and decode throughput of a Gadopel model at layer sizes of a served model (random weights), beside
+a Llama model of equal width, depth, feed-forward and vocabulary, with the device time per class
+of kernel of one decode step and one prefill of each.
 """
 import argparse
 import json
@@ -63,8 +70,116 @@ def prefill_flops(cfg, T):
     return linear + attn + 2 * V * H
 
 
+# --design gadopel: layers of width 2,048 with a feed-forward of 8,192.  Latent layers with 16
+# heads of 128 + 64 query/key elements over rows of 512 + 64, windowed layers with 32 heads of 64
+# over 8 kv heads and a window of 1,024 that keeps 64 first positions, in turn; the Llama beside it
+# has 32 heads of 64 over 8 kv heads in every layer.
+def gadopel_config(layers: int, vocab: int) -> dict:
+    latent = {"type": "latent_attention", "mlp": {"kind": "dense", "ff": 8192},
+              "mixer": {"heads": 16, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512, "scale": 192 ** -0.5,
+                        "rot": {"base": 10000.0, "dims": 64}}}
+    windowed = {"type": "attention", "mlp": {"kind": "dense", "ff": 8192},
+                "mixer": {"heads": 32, "kv_heads": 8, "dim": 64, "vdim": 64, "scale": 1.0,
+                          "mask": {"size": 1024, "keep_first": 64},
+                          "rot": {"base": 500000.0, "dims": 64,
+                                  "scaling": {"factor": 8.0, "original": 2048, "fast": 32.0, "slow": 1.0}}}}
+    return {"architecture": "Gadopel", "vocab": vocab, "width": 2048, "norm": {"eps": 1e-6},
+            "layers": [latent if i % 2 == 0 else windowed for i in range(layers)], "max_positions": 8192}
+
+
+def design_comparison(args) -> int:
+    import torch
+    from kv_cache_optimization_for_llm_amd.engine.batch import StepEntry
+    from kv_cache_optimization_for_llm_amd.engine.engine import Engine, EngineOptions
+    from kv_cache_optimization_for_llm_amd.ops import kernels as K
+
+    layers, vocab = args.layers or 8, 32000
+    llama = dict(CONFIG_1B, num_hidden_layers=layers, vocab_size=vocab, tie_word_embeddings=False)
+    configs = {"gadopel": gadopel_config(layers, vocab), "llama": llama}
+    shapes = [(8, 4096), (32, 2048)]            # (requests, context) of the decode runs
+    gen = torch.Generator().manual_seed(0)
+    out = {}
+    for name, cfg in configs.items():
+        pool = max(b * (c + 2 * PAGE) for b, c in shapes)
+        engine = Engine(None, EngineOptions(dtype="bfloat16", page_size=PAGE, cache_tokens=pool, max_seqs=32,
+                                            max_seq_len=8192, max_batch_tokens=8192, max_logit_rows=64),
+                        config_dict=cfg, random_seed=0)
+        res = {"weight_gb": round(sum(t.numel() * t.element_size() for t in
+                                      [lin.weight for lin in engine.model.linears()]) / 1e9, 3),
+               "cache_bytes_per_token": engine.cache.page_bytes() // PAGE}
+
+        def timed_prefill(tokens):
+            prompt = [int(t) for t in torch.randint(0, vocab, (tokens,), generator=gen)]
+            best = 1e9
+            for i in range(5):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                engine.step([StepEntry(f"p{i}", prompt, [tokens - 1])])
+                torch.cuda.synchronize()
+                best = min(best, time.perf_counter() - t0) if i else best
+                engine.release(f"p{i}")
+            return best
+
+        for tokens in (PREFILL_TOKENS,):
+            sec = timed_prefill(tokens)
+            res[f"prefill_{tokens}_tok_s"] = round(tokens / sec, 1)
+            res[f"prefill_{tokens}_ms"] = round(sec * 1e3, 3)
+        for batch, context in shapes:
+            ids = [f"d{i}" for i in range(batch)]
+            base = [int(t) for t in torch.randint(0, vocab, (context - args.steps - args.warmup - 4,), generator=gen)]
+            for rid in ids:
+                for lo in range(0, len(base), 4096):
+                    engine.step([StepEntry(rid, base[lo:lo + 4096], [])])
+            step = [StepEntry(rid, [7], [0]) for rid in ids]
+            for _ in range(args.warmup + 2):
+                engine.step(step)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                engine.step(step)
+            torch.cuda.synchronize()
+            sec = time.perf_counter() - t0
+            res[f"decode_b{batch}_c{context}_tok_s"] = round(batch * args.steps / sec, 1)
+            res[f"decode_b{batch}_c{context}_ms"] = round(sec / args.steps * 1e3, 4)
+            if (batch, context) == shapes[0]:
+                graphs, portion_graphs = engine.graphs, engine.portion_graphs
+                engine.graphs = engine.portion_graphs = None        # launched one by one, events between
+                engine.step(step)
+                with K.KernelClassTimer() as timer:
+                    engine.step(step)
+                res[f"kclass_decode_b{batch}_c{context}_ms"] = timer.milliseconds()
+                engine.graphs, engine.portion_graphs = graphs, portion_graphs
+            for rid in ids:
+                engine.release(rid)
+        graphs, portion_graphs = engine.graphs, engine.portion_graphs
+        engine.graphs = engine.portion_graphs = None
+        prompt = [int(t) for t in torch.randint(0, vocab, (PREFILL_TOKENS,), generator=gen)]
+        engine.step([StepEntry("kp0", prompt, [PREFILL_TOKENS - 1])])
+        engine.release("kp0")
+        with K.KernelClassTimer() as timer:
+            engine.step([StepEntry("kp1", prompt, [PREFILL_TOKENS - 1])])
+        res[f"kclass_prefill_{PREFILL_TOKENS}_ms"] = timer.milliseconds()
+        engine.release("kp1")
+        out[name] = res
+        del engine
+        import gc
+        gc.collect()
+        torch.cuda.empty_cache()
+    b, c = shapes[0]
+    print(json.dumps({"metric": "gadopel_decode_tokens_per_second", "value": out["gadopel"][f"decode_b{b}_c{c}_tok_s"],
+                      "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+                      "higher_is_better": True, "dtype": "bf16", "data": "synthetic (random weights, seeded token ids)",
+                      "config": {"design": "gadopel beside llama", "layers": layers, "width": 2048, "ff": 8192,
+                                 "vocab": vocab, "decode_shapes": shapes, "prefill_tokens": PREFILL_TOKENS},
+                      "designs": out}))
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--design", choices=["gadopel"], default=None,
+                    help="another measurement (its own JSON line): a model of this design at the layer sizes of a "
+                         "served model beside a Llama model of equal size; the default run is left as it is")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=16)
@@ -83,6 +198,8 @@ def main():
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on a single MI355X)")
         return 2
+    if args.design:
+        return design_comparison(args)
 
     import torch
     from kv_cache_optimization_for_llm_amd.engine.batch import StepEntry

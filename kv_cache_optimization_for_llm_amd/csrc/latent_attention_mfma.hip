@@ -247,3 +247,219 @@ extern "C" int kva_latent_attention_mfma(void *out, float *part_o, float *part_m
     }
     return KVA_OK;
 }
+
+
+// ---- grouped-query attention with the same options ---------------------------------------------
+//
+// The kernel above over the paged K / V^T arrays of ordinary attention (kv_layout.h), for what the
+// tuned kernels of attention_mfma.hip do not take: a window that keeps a request's first
+// positions visible, a sink per head, values of another size than the keys.  Rows of a tile are
+// (token, query head of the kv head's group) pairs, row = token_in_entry * G + head_in_group; one
+// wavefront per (item, kv head, key range).  D = 32 NKS key elements, DV = 16 NDT value elements.
+template <int NDT, int NKS>
+__global__ void __launch_bounds__(KVA_WAVE)
+gqa_attention_rows_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_ml,
+                          const bf16_t *__restrict__ q, int q_stride, const bf16_t *__restrict__ k_cache,
+                          const bf16_t *__restrict__ v_cache, const int *__restrict__ block_table, int max_blocks,
+                          const int *__restrict__ item_entry, const int *__restrict__ item_row0,
+                          const int *__restrict__ entry_seat, const int *__restrict__ entry_q_start,
+                          const int *__restrict__ entry_start_pos, int heads, int kv_heads, int page_size,
+                          float scale, int window, int keep_first, const float *__restrict__ sinks, int splits,
+                          int per_split) {
+    constexpr int DV = NDT * 16, D = NKS * 32;
+    const int lane = threadIdx.x, r = lane & 15, g = lane >> 4;
+    const int item = blockIdx.x, kvh = blockIdx.y / splits, split = blockIdx.y % splits;
+    const int group = heads / kv_heads;
+    const int e = item_entry[item], row0 = item_row0[item];
+    const int q_start = entry_q_start[e], q_len = entry_q_start[e + 1] - q_start;
+    const int start_pos = entry_start_pos[e];
+    const int *bt = block_table + (size_t)entry_seat[e] * max_blocks;
+    const int rows = q_len * group;
+    if (row0 >= rows) return;
+    const int last_row = min(row0 + 15, rows - 1);
+    const int item_hi = start_pos + last_row / group;
+    const int pos_lo = start_pos + row0 / group;
+    const int my_row = min(row0 + r, rows - 1);
+    const bool row_valid = row0 + r < rows;
+    const int my_pos = start_pos + my_row / group;
+    const int my_head = kvh * group + my_row % group;
+    const int my_lo = (window > 0 && my_pos - window + 1 > 0) ? my_pos - window + 1 : 0;
+    const int item_lo = (window > 0 && pos_lo - window + 1 > 0) ? pos_lo - window + 1 : 0;
+    const size_t my_token = (size_t)q_start + my_row / group;
+
+    Frag8 qf[NKS];
+    {
+        const bf16_t *qrow = q + my_token * q_stride + (size_t)my_head * D + 8 * g;
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) qf[ks].u4 = *reinterpret_cast<const uint4 *>(qrow + 32 * ks);
+    }
+    f32x4 o[NDT];
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.f;
+    const float scale2 = scale * LAT_LOG2E;
+
+    int k_begin = 0, k_end = item_hi + 1;
+    if (splits > 1) {
+        k_begin = split * per_split;
+        k_end = min(k_end, k_begin + per_split);
+    }
+    for (int kstart = k_begin & ~31; kstart < k_end; kstart += 32) {
+        if (kstart + 32 <= item_lo && kstart >= keep_first) continue;
+        int page[2];
+        bool mapped[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int key0 = kstart + 16 * t;
+            const int p = key0 <= item_hi ? bt[key0 / page_size] : -1;
+            mapped[t] = p >= 0;
+            page[t] = p >= 0 ? p : 0;
+        }
+        f32x4 s[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int key = kstart + 16 * t + r;
+            // K pages are [D / 8][page_size][8]: chunk 4 ks + g of key `key`
+            const bf16_t *kp = k_cache + ((size_t)page[t] * kv_heads + kvh) * page_size * D +
+                               ((size_t)g * page_size + key % page_size) * 8;
+            s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks) {
+                Frag8 kf;
+                kf.u4 = *reinterpret_cast<const uint4 *>(kp + (size_t)ks * 4 * page_size * 8);
+                s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[ks].v, s[t], 0, 0, 0);
+            }
+        }
+        float sv[8], mx = -INFINITY;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int key = kstart + 16 * t + 4 * g + i;
+                const bool vis = row_valid && mapped[t] && key <= my_pos && (key >= my_lo || key < keep_first) &&
+                                 key >= k_begin && key < k_end;
+                const float x = vis ? s[t][i] * scale2 : -INFINITY;
+                sv[t * 4 + i] = x;
+                mx = fmaxf(mx, x);
+            }
+        const float m_new = fmaxf(m, quad_rows_max(mx));
+        const float ref = (m_new == -INFINITY) ? 0.f : m_new;
+        const float corr = __builtin_amdgcn_exp2f(m - ref);
+        l *= corr;
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt) {
+            o[dt][0] *= corr; o[dt][1] *= corr; o[dt][2] *= corr; o[dt][3] *= corr;
+        }
+        m = m_new;
+        Frag8 pf;
+#pragma unroll
+        for (int j = 0; j < 8; j += 2) {
+            const float p0 = __builtin_amdgcn_exp2f(sv[j] - ref), p1 = __builtin_amdgcn_exp2f(sv[j + 1] - ref);
+            l += p0 + p1;
+            pf.p2[j / 2] = pack_bf16(p0, p1);
+        }
+        uint2 keep[2];
+        const bf16_t *vrow[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int key0 = kstart + 16 * t + 4 * g;
+            int n = min(item_hi + 1, k_end) - key0;
+            if (!mapped[t] || key0 + 4 <= k_begin) n = 0;
+            keep[t] = keep_first_keys(make_uint2(~0u, ~0u), n);
+            if (key0 < k_begin && n > 0) {
+                const uint2 head = keep_first_keys(make_uint2(~0u, ~0u), k_begin - key0);
+                keep[t].x &= ~head.x; keep[t].y &= ~head.y;
+            }
+            vrow[t] = v_cache + (((size_t)page[t] * kv_heads + kvh) * DV + r) * page_size + key0 % page_size;
+        }
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt) {
+            Frag8 vv;
+            vv.u2[0] = *reinterpret_cast<const uint2 *>(vrow[0] + (size_t)dt * 16 * page_size);
+            vv.u2[1] = *reinterpret_cast<const uint2 *>(vrow[1] + (size_t)dt * 16 * page_size);
+            vv.u2[0].x &= keep[0].x; vv.u2[0].y &= keep[0].y;
+            vv.u2[1].x &= keep[1].x; vv.u2[1].y &= keep[1].y;
+            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv.v, pf.v, o[dt], 0, 0, 0);
+        }
+    }
+    l = quad_rows_sum(l);
+    if (!row_valid) return;
+    const size_t my_global = my_token * heads + my_head;           // row of the output, of the partial results
+    if (splits > 1) {
+        float *po = part_o + (my_global * splits + split) * DV + 4 * g;
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt) *reinterpret_cast<float4 *>(po + 16 * dt) = make_float4(o[dt][0], o[dt][1], o[dt][2], o[dt][3]);
+        if (g == 0) {
+            part_ml[(my_global * splits + split) * 2] = m;
+            part_ml[(my_global * splits + split) * 2 + 1] = l;
+        }
+        return;
+    }
+    float mul = 1.f;
+    if (sinks) {
+        const float sk = sinks[my_head] * LAT_LOG2E, m_new = fmaxf(m, sk);
+        const float corr = __builtin_amdgcn_exp2f(m - m_new);
+        l = l * corr + __builtin_amdgcn_exp2f(sk - m_new);
+        mul = corr;
+    }
+    mul /= l;
+    bf16_t *orow = out + my_global * DV + 4 * g;
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) {
+        Frag4 w;
+        w.h[0] = float_to_bf16_bits(o[dt][0] * mul); w.h[1] = float_to_bf16_bits(o[dt][1] * mul);
+        w.h[2] = float_to_bf16_bits(o[dt][2] * mul); w.h[3] = float_to_bf16_bits(o[dt][3] * mul);
+        *reinterpret_cast<uint2 *>(orow + 16 * dt) = w.u2;
+    }
+}
+
+// (value size / 16, key size / 32) pairs with an instance
+#define GQA_ROWS_INSTANCES(X) X(2, 1) X(4, 1) X(2, 2) X(4, 2) X(8, 2) X(6, 3) X(4, 4) X(8, 4) X(12, 6) X(16, 8)
+
+extern "C" int kva_attention_rows_mfma_supported(int head_dim, int value_dim, int page_size) {
+    if (page_size <= 0 || page_size % 16) return 0;
+#define CHECK_ONE(NDT, NKS) if (value_dim == NDT * 16 && head_dim == NKS * 32) return 1;
+    GQA_ROWS_INSTANCES(CHECK_ONE)
+#undef CHECK_ONE
+    return 0;
+}
+
+extern "C" int kva_attention_rows_mfma(void *out, float *part_o, float *part_ml, const void *q, int q_stride,
+                                       const void *k_cache, const void *v_cache, const int *block_table,
+                                       int max_blocks, const int *item_entry, const int *item_row0,
+                                       const int *entry_seat, const int *entry_q_start, const int *entry_start_pos,
+                                       int num_items, int total_rows, int heads, int kv_heads, int head_dim,
+                                       int value_dim, int page_size, float scale, int window, int keep_first,
+                                       const float *sinks, int splits, int per_split, hipStream_t stream) {
+    KVA_REQUIRE(kva_attention_rows_mfma_supported(head_dim, value_dim, page_size),
+                "attention_rows_mfma: no instance for keys of %d, values of %d, pages of %d", head_dim, value_dim, page_size);
+    KVA_REQUIRE(num_items >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && max_blocks > 0 && total_rows >= 0,
+                "attention_rows_mfma: bad sizes");
+    KVA_REQUIRE(q_stride % 8 == 0 && q_stride >= heads * head_dim, "attention_rows_mfma: query row stride %d", q_stride);
+    KVA_REQUIRE(splits >= 1 && (long long)splits * kv_heads <= 65535 &&
+                    (splits == 1 || (per_split > 0 && per_split % 32 == 0 && part_o && part_ml)),
+                "attention_rows_mfma: key ranges need a length that is a multiple of 32 and a workspace");
+    KVA_REQUIRE(window >= 0 && keep_first >= 0, "attention_rows_mfma: negative window or kept first positions");
+    if (window == 0) keep_first = 0;
+    if (num_items == 0) return KVA_OK;
+    dim3 grid(num_items, kv_heads * splits), block(KVA_WAVE);
+    bool done = false;
+#define LAUNCH_ONE(NDT, NKS)                                                                                    \
+    if (!done && value_dim == NDT * 16 && head_dim == NKS * 32) {                                               \
+        hipLaunchKernelGGL((gqa_attention_rows_kernel<NDT, NKS>), grid, block, 0, stream, (bf16_t *)out, part_o, \
+                           part_ml, (const bf16_t *)q, q_stride, (const bf16_t *)k_cache,                        \
+                           (const bf16_t *)v_cache, block_table, max_blocks, item_entry, item_row0, entry_seat,  \
+                           entry_q_start, entry_start_pos, heads, kv_heads, page_size, scale, window,            \
+                           keep_first, sinks, splits, per_split);                                                \
+        done = true;                                                                                             \
+    }
+    GQA_ROWS_INSTANCES(LAUNCH_ONE)
+#undef LAUNCH_ONE
+    KVA_CHECK_LAUNCH("attention_rows_mfma");
+    if (splits > 1) {
+        hipLaunchKernelGGL(latent_merge_kernel, dim3(total_rows), dim3(256), 0, stream, (bf16_t *)out, part_o, part_ml,
+                           sinks, heads, value_dim, splits);
+        KVA_CHECK_LAUNCH("attention_rows_merge");
+    }
+    return KVA_OK;
+}

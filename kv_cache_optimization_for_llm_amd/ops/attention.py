@@ -366,7 +366,8 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
 
     ``keep_first`` (with a window: the first so many positions stay visible behind it), ``sinks``
     (fp32 per query head: one more term exp(sink) in every denominator) and a ``value_dim`` other
-    than ``head_dim`` are taken by the plain kernel only."""
+    than ``head_dim`` are taken by a matrix-core kernel of their own (16 rows of (token, head)
+    pairs a wavefront; bf16, head sizes with an instance) or else by the plain kernel."""
     if kv is None:
         raise K.KernelError("paged_attention: the mixer has no cache view")
     value_dim = head_dim if value_dim is None else int(value_dim)
@@ -376,6 +377,16 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
         if rope is not None or max_parts:
             raise K.KernelError("paged_attention: kept first positions, sinks and a value size of its own "
                                 "go with neither rotation inside the kernel nor partial results")
+        if qkv.dtype == torch.bfloat16 and qkv.shape[1] % 8 == 0 \
+                and K.attention_rows_mfma_supported(head_dim, value_dim, kv.page_size):
+            from .latent_attention import choose_ranges
+            item_entry, item_row0, _ = batch.attention_items(num_q_heads // num_kv_heads, 1, "all")
+            # a window bounds what a row reads whatever the context: its keys are not cut into ranges
+            ranges, per = (1, 0) if window > 0 else choose_ranges(item_entry.shape[0] * num_kv_heads, batch.max_context)
+            return K.attention_rows_mfma(qkv, qkv.shape[1], out, kv.k_cache, kv.v_cache, kv.block_table, item_entry,
+                                         item_row0, batch.entry_seat, batch.entry_q_start, batch.entry_start_pos,
+                                         num_q_heads, num_kv_heads, head_dim, scale, window, keep_first, sinks,
+                                         value_dim, ranges, per)
         return K.attention_rowwise(qkv, qkv.shape[1], out, kv.k_cache, kv.v_cache, kv.block_table,
                                    batch.tok_seat, batch.positions, num_q_heads, num_kv_heads,
                                    head_dim, scale, window, keep_first, sinks, value_dim)

@@ -467,6 +467,53 @@ def latent_attention_mfma(q: torch.Tensor, out: torch.Tensor, cache: torch.Tenso
     return out
 
 
+def attention_rows_mfma_supported(head_dim: int, value_dim: int, page_size: int) -> bool:
+    return bool(hip_lib().kva_attention_rows_mfma_supported(int(head_dim), int(value_dim), int(page_size)))
+
+
+def attention_rows_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_cache: torch.Tensor,
+                        v_cache: torch.Tensor, block_table: torch.Tensor, item_entry: torch.Tensor,
+                        item_row0: torch.Tensor, entry_seat: torch.Tensor, entry_q_start: torch.Tensor,
+                        entry_start_pos: torch.Tensor, num_q_heads: int, num_kv_heads: int, head_dim: int,
+                        scale: float, window: int = 0, keep_first: int = 0, sinks: Optional[torch.Tensor] = None,
+                        value_dim: Optional[int] = None, splits: int = 1, per_split: int = 0) -> torch.Tensor:
+    """:func:`attention_rowwise` with all its options on the matrix cores (bf16): a work item is 16
+    rows ``token_in_entry * group + head_in_group`` of entry ``item_entry[i]`` from ``item_row0[i]``
+    on, for every kv head; with ``splits`` > 1 the keys are cut into ranges of ``per_split`` and a
+    second kernel adds the ranges' results up."""
+    tokens = out.shape[0]
+    value_dim = head_dim if value_dim is None else int(value_dim)
+    if out.shape != (tokens, num_q_heads * value_dim):
+        raise KernelError("attention_rows_mfma: out must be [T, nq * value size]")
+    page_size = check_kv_cache_shapes("attention_rows_mfma", k_cache, v_cache, num_kv_heads, head_dim, value_dim)
+    if not (q.dtype == out.dtype == k_cache.dtype == v_cache.dtype == torch.bfloat16):
+        raise KernelError("attention_rows_mfma: bfloat16 only")
+    if not attention_rows_mfma_supported(head_dim, value_dim, page_size):
+        raise KernelError(f"attention_rows_mfma: no instance for keys of {head_dim}, values of {value_dim}, pages of {page_size}")
+    if q.data_ptr() % 16 or q_row_stride < num_q_heads * head_dim or q_row_stride % 8:
+        raise KernelError("attention_rows_mfma: q view is misaligned or its stride does not fit")
+    n, entries = item_entry.shape[0], entry_seat.shape[0]
+    if item_row0.shape != (n,) or entry_q_start.shape != (entries + 1,) or entry_start_pos.shape != (entries,):
+        raise KernelError("attention_rows_mfma: one row0 per item, entries + 1 starts, one start position per entry")
+    if sinks is not None and (sinks.shape != (num_q_heads,) or sinks.dtype != torch.float32):
+        raise KernelError("attention_rows_mfma: sinks are fp32, one per query head")
+    part_o = part_ml = None
+    if splits > 1:
+        if per_split <= 0 or per_split % 32:
+            raise KernelError("attention_rows_mfma: key ranges are multiples of 32 keys")
+        part_o = torch.empty((tokens * num_q_heads, splits, value_dim), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((tokens * num_q_heads, splits, 2), dtype=torch.float32, device=q.device)
+    check(hip_lib().kva_attention_rows_mfma(
+        _dev(out, "out"), _opt(part_o, "part_o"), _opt(part_ml, "part_ml"), _dev(q, "q", contiguous=False), q_row_stride,
+        _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"), _dev(block_table, "block_table", torch.int32),
+        block_table.shape[1], _dev(item_entry, "item_entry", torch.int32), _dev(item_row0, "item_row0", torch.int32),
+        _dev(entry_seat, "entry_seat", torch.int32), _dev(entry_q_start, "entry_q_start", torch.int32),
+        _dev(entry_start_pos, "entry_start_pos", torch.int32), n, tokens * num_q_heads, num_q_heads, num_kv_heads,
+        head_dim, value_dim, page_size, float(scale), int(window), int(keep_first), _opt(sinks, "sinks"), int(splits),
+        int(per_split), _stream()), "attention_rows_mfma")
+    return out
+
+
 def layernorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor, deltas=(),
               row_idx: Optional[torch.Tensor] = None, weight2: Optional[torch.Tensor] = None,
               out2: Optional[torch.Tensor] = None, rms: bool = False) -> torch.Tensor:
@@ -1294,6 +1341,10 @@ KERNEL_CLASSES = {
     "residual_add": "elementwise", "scale_softcap": "elementwise", "cast": "elementwise",
     "silu_mul": "activation", "rope_kv_write": "rope + cache write",
     "attention_rowwise": "attention", "attention_mfma": "attention", "attention_lds": "attention",
+    "attention_rows_mfma": "attention", "latent_attention_rowwise": "attention", "latent_attention_mfma": "attention",
+    "layernorm": "norm", "stream_join": "elementwise", "head_gate": "elementwise", "act_mul": "activation",
+    "qk_encode_cache": "rope + cache write", "latent_encode_cache": "rope + cache write",
+    "heads_matmul": "per-head products",
     "attention_mfma_rope": "attention",
     "gemm_nt_f32": "gemm fp32", "gemm_vendor": "gemm (vendor library)",
     "gemm_skinny": "gemm (few rows)", "gemm_skinny_qkv_rope": "gemm (few rows)",

@@ -291,3 +291,39 @@ def test_latent_attention_on_the_matrix_cores(heads, rank, rot, window, keep_fir
                                 ranges, per_range)
         assert torch.isfinite(out.float()).all(), f"entry {start}+{n}"
         close(out, want_all[start:upto], 3e-2, f"entry {start}+{n}")
+
+
+@pytest.mark.parametrize("per_range", [0, 64])
+@pytest.mark.parametrize("heads, kv_heads, dim, vdim, window, keep_first", [
+    (4, 1, 64, 64, 40, 20), (8, 2, 32, 64, 33, 17), (6, 3, 64, 32, 0, 0), (32, 2, 64, 64, 16, 16), (2, 2, 128, 128, 50, 0)])
+def test_windowed_attention_on_the_matrix_cores(heads, kv_heads, dim, vdim, window, keep_first, per_range, gpu):
+    """The matrix-core kernel that takes a window with kept first positions, sinks and a value
+    size of its own: portions of prompts and decoded tokens against the plain attention."""
+    page, scale, length = 16, 0.2, 200
+    assert K.attention_rows_mfma_supported(dim, vdim, page)
+    group = heads // kv_heads
+    q_all = rnd((length, heads, dim), 31, torch.bfloat16)
+    k_all, v_all = rnd((length, kv_heads, dim), 32, torch.bfloat16), rnd((length, kv_heads, vdim), 33, torch.bfloat16)
+    sinks = rnd((heads,), 34) * 2
+    table, slots, pages = cache_for(length, page, 19)
+    prob = plain.softmax_rows(torch.einsum("ihd,jhd->hij", q_all.double(), k_all.double().repeat_interleave(group, dim=1)) * scale,
+                              plain.visible(length, window, keep_first), sinks.double())
+    want_all = torch.einsum("hij,jhd->ihd", prob, v_all.double().repeat_interleave(group, dim=1))
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=gpu)
+    for start, n in [(37, 30), (199, 1), (0, 9), (112, 1), (96, 16)]:
+        upto = start + n
+        kp = torch.full((pages, kv_heads, page, dim), float("nan"), dtype=torch.bfloat16, device=gpu)
+        v_cache = torch.full((pages, kv_heads, vdim, page), float("nan"), dtype=torch.bfloat16, device=gpu)
+        sl = slots[:upto].long().to(gpu)
+        kp[sl // page, :, sl % page] = k_all[:upto].to(gpu)
+        v_cache[sl // page, :, :, sl % page] = v_all[:upto].to(gpu)
+        k_cache = K.keys_to_pages(kp)
+        q = q_all[start:upto].reshape(n, heads * dim).contiguous().to(gpu)
+        tiles = (n * group + 15) // 16
+        out = torch.empty((n, heads * vdim), dtype=torch.bfloat16, device=gpu)
+        ranges = 1 if per_range == 0 else -(-upto // per_range)
+        K.attention_rows_mfma(q, heads * dim, out, k_cache, v_cache, table.to(gpu), i32([0] * tiles),
+                              i32([16 * t for t in range(tiles)]), i32([1]), i32([0, n]), i32([start]), heads, kv_heads,
+                              dim, scale, window, keep_first, sinks.to(gpu), vdim, ranges, per_range)
+        assert torch.isfinite(out.float()).all(), f"entry {start}+{n}"
+        close(out.view(n, heads, vdim), want_all[start:upto], 3e-2, f"entry {start}+{n}")
