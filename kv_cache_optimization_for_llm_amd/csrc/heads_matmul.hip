@@ -85,3 +85,90 @@ extern "C" int kva_heads_matmul(void *out, int o_row, int o_head, const void *x,
     KVA_CHECK_LAUNCH("heads_matmul");
     return KVA_OK;
 }
+
+// ---- the same product on the matrix cores (bf16) ------------------------------------------------
+//
+// A wavefront takes 16 outputs n of one head and walks over tiles of 16 rows t:
+// out^T[n, t] = W[h][n, :] . x[t, h, :].  A = 16 rows of W[h] (16 bytes a lane, row-major), kept
+// in registers for all the row tiles the wavefront visits; B = x^T: lane (row t, group g) loads 16
+// bytes of its row.  K = 32 NKS.  blockIdx: (n tile, head, group of row tiles).
+#include "attention_frag.h"
+
+template <int NKS>
+__global__ void __launch_bounds__(KVA_WAVE)
+heads_matmul_mfma_kernel(bf16_t *__restrict__ out, int o_row, int o_head, const bf16_t *__restrict__ x, int x_row,
+                         int x_head, const bf16_t *__restrict__ w, int M, int N, int tiles_per_wave) {
+    constexpr int K = NKS * 32;
+    const int lane = threadIdx.x, r = lane & 15, g = lane >> 4;
+    const int n0 = blockIdx.x * 16, h = blockIdx.y;
+    Frag8 wf[NKS];
+    {
+        const int n = min(n0 + r, N - 1);
+        const bf16_t *wrow = w + ((size_t)h * N + n) * K + 8 * g;
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) wf[ks].u4 = *reinterpret_cast<const uint4 *>(wrow + 32 * ks);
+    }
+    const int first = blockIdx.z * tiles_per_wave;
+    for (int tile = first; tile < first + tiles_per_wave && tile * 16 < M; ++tile) {
+        const int t = min(tile * 16 + r, M - 1);
+        const bf16_t *xrow = x + (size_t)t * x_row + (size_t)h * x_head + 8 * g;
+        f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) {
+            Frag8 xf;
+            xf.u4 = *reinterpret_cast<const uint4 *>(xrow + 32 * ks);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[ks].v, xf.v, acc, 0, 0, 0);
+        }
+        // lane (row t = r, group g) holds outputs n0 + 4 g .. + 3 of its row
+        if (tile * 16 + r < M) {
+            bf16_t *o = out + (size_t)t * o_row + (size_t)h * o_head + n0 + 4 * g;
+            if (n0 + 4 * g + 3 < N && ((o_row | o_head) % 4 == 0)) {
+                Frag4 v;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) v.h[i] = float_to_bf16_bits(acc[i]);
+                *reinterpret_cast<uint2 *>(o) = v.u2;
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (n0 + 4 * g + i < N) o[i].bits = float_to_bf16_bits(acc[i]);
+            }
+        }
+    }
+}
+
+#define HM_INSTANCES(X) X(1) X(2) X(3) X(4) X(6) X(8) X(12) X(16)
+
+extern "C" int kva_heads_matmul_mfma_supported(int K, int x_row, int x_head) {
+    if (K % 32 || x_row % 8 || x_head % 8) return 0;
+#define CHECK_ONE(NKS) if (K == NKS * 32) return 1;
+    HM_INSTANCES(CHECK_ONE)
+#undef CHECK_ONE
+    return 0;
+}
+
+extern "C" int kva_heads_matmul_mfma(void *out, int o_row, int o_head, const void *x, int x_row, int x_head,
+                                     const void *w, int rows, int heads, int N, int K, hipStream_t stream) {
+    KVA_REQUIRE(rows >= 0 && heads > 0 && heads <= 65535 && N > 0, "heads_matmul_mfma: bad sizes");
+    KVA_REQUIRE(kva_heads_matmul_mfma_supported(K, x_row, x_head),
+                "heads_matmul_mfma: no instance for K = %d with strides %d / %d", K, x_row, x_head);
+    KVA_REQUIRE(x_head >= K && o_head >= N && x_row >= (heads - 1) * x_head + K && o_row >= (heads - 1) * o_head + N,
+                "heads_matmul_mfma: strides do not fit %d heads of %d -> %d", heads, K, N);
+    if (rows == 0) return KVA_OK;
+    const int row_tiles = (rows + 15) / 16;
+    // enough wavefronts to fill the chip before a wavefront takes more than one row tile
+    int per_wave = 1;
+    while (per_wave < 8 && (long long)((N + 15) / 16) * heads * ((row_tiles + per_wave - 1) / per_wave) > 4096) per_wave *= 2;
+    dim3 grid((N + 15) / 16, heads, (row_tiles + per_wave - 1) / per_wave), block(KVA_WAVE);
+    KVA_REQUIRE(grid.z <= 65535, "heads_matmul_mfma: %d rows are too many for one launch", rows);
+    bool done = false;
+#define LAUNCH_ONE(NKS)                                                                                          \
+    if (!done && K == NKS * 32) {                                                                                \
+        hipLaunchKernelGGL(heads_matmul_mfma_kernel<NKS>, grid, block, 0, stream, (bf16_t *)out, o_row, o_head,  \
+                           (const bf16_t *)x, x_row, x_head, (const bf16_t *)w, rows, N, per_wave);              \
+        done = true;                                                                                             \
+    }
+    HM_INSTANCES(LAUNCH_ONE)
+#undef LAUNCH_ONE
+    KVA_CHECK_LAUNCH("heads_matmul_mfma");
+    return KVA_OK;
+}

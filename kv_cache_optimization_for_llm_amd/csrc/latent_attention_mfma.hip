@@ -23,9 +23,13 @@
 
 #define LAT_LOG2E 1.44269504088896340736f
 
+// The body; two kernels below give it one or up to four wavefronts a SIMD.  A block's loads are
+// all asked for before its first product (a load inside the product loop compiles to one trip to
+// memory per product): the 2 NKS key fragments at once, the value fragments eight tiles ahead.
+// The queries wait in LDS (one wavefront's 16 rows), so that the registers hold the keys in flight.
 template <int NDT /* RANK / 16 */, int NKS /* KD / 32 */>
-__global__ void __launch_bounds__(KVA_WAVE)
-latent_attention_mfma_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_ml,
+__device__ __forceinline__ void
+latent_attention_mfma_body(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_ml,
                              const bf16_t *__restrict__ q, const bf16_t *__restrict__ cache,
                              const bf16_t *__restrict__ cache_t, const int *__restrict__ block_table, int max_blocks,
                              const int *__restrict__ item_entry, const int *__restrict__ item_row0,
@@ -50,12 +54,13 @@ latent_attention_mfma_kernel(bf16_t *__restrict__ out, float *__restrict__ part_
     const int item_lo = (window > 0 && pos_lo - window + 1 > 0) ? pos_lo - window + 1 : 0;
     const size_t my_global = (size_t)q_start * heads + my_row;      // row of q / out
 
-    // Q^T in operand layout: lane (row r, group g) holds elements 32 ks + 8 g .. + 7 of its row
-    Frag8 qf[NKS];
+    // Q^T in operand layout: lane (row r, group g) holds elements 32 ks + 8 g .. + 7 of its row;
+    // kept in LDS as [ks][lane] (a lane reads back what it wrote: no barrier)
+    __shared__ uint4 q_s[NKS * KVA_WAVE];
     {
         const bf16_t *qrow = q + my_global * KD + 8 * g;
 #pragma unroll
-        for (int ks = 0; ks < NKS; ++ks) qf[ks].u4 = *reinterpret_cast<const uint4 *>(qrow + 32 * ks);
+        for (int ks = 0; ks < NKS; ++ks) q_s[ks * KVA_WAVE + lane] = *reinterpret_cast<const uint4 *>(qrow + 32 * ks);
     }
     f32x4 o[NDT];
 #pragma unroll
@@ -82,16 +87,23 @@ latent_attention_mfma_kernel(bf16_t *__restrict__ out, float *__restrict__ part_
             page[t] = p >= 0 ? p : 0;                       // a tile nobody sees is read from a page that exists
         }
         f32x4 s[2];
+        Frag8 kf[2][NKS];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             const int key = kstart + 16 * t + r;
             const bf16_t *krow = cache + ((size_t)page[t] * page_size + key % page_size) * KD + 8 * g;
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks) kf[t][ks].u4 = *reinterpret_cast<const uint4 *>(krow + 32 * ks);
+        }
+        __builtin_amdgcn_sched_barrier(0);              // every key load of the block is out before the first product
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
             s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int ks = 0; ks < NKS; ++ks) {
-                Frag8 kf;
-                kf.u4 = *reinterpret_cast<const uint4 *>(krow + 32 * ks);
-                s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[ks].v, s[t], 0, 0, 0);
+                Frag8 qf;
+                qf.u4 = q_s[ks * KVA_WAVE + lane];
+                s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t][ks].v, qf.v, s[t], 0, 0, 0);
             }
         }
         // mask and online softmax: lane (row r, group g) holds keys kstart + 16 t + 4 g + i
@@ -141,14 +153,22 @@ latent_attention_mfma_kernel(bf16_t *__restrict__ out, float *__restrict__ part_
             }
             vrow[t] = cache_t + ((size_t)page[t] * RANK + r) * page_size + key0 % page_size;
         }
+        constexpr int VC = NDT < 8 ? NDT : 8;                          // value tiles asked for together
 #pragma unroll
-        for (int dt = 0; dt < NDT; ++dt) {
-            Frag8 vv;
-            vv.u2[0] = *reinterpret_cast<const uint2 *>(vrow[0] + (size_t)dt * 16 * page_size);
-            vv.u2[1] = *reinterpret_cast<const uint2 *>(vrow[1] + (size_t)dt * 16 * page_size);
-            vv.u2[0].x &= keep[0].x; vv.u2[0].y &= keep[0].y;
-            vv.u2[1].x &= keep[1].x; vv.u2[1].y &= keep[1].y;
-            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv.v, pf.v, o[dt], 0, 0, 0);
+        for (int d0 = 0; d0 < NDT; d0 += VC) {
+            Frag8 vv[VC];
+#pragma unroll
+            for (int j = 0; j < VC; ++j) {
+                vv[j].u2[0] = *reinterpret_cast<const uint2 *>(vrow[0] + (size_t)(d0 + j) * 16 * page_size);
+                vv[j].u2[1] = *reinterpret_cast<const uint2 *>(vrow[1] + (size_t)(d0 + j) * 16 * page_size);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < VC; ++j) {
+                vv[j].u2[0].x &= keep[0].x; vv[j].u2[0].y &= keep[0].y;
+                vv[j].u2[1].x &= keep[1].x; vv[j].u2[1].y &= keep[1].y;
+                o[d0 + j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv[j].v, pf.v, o[d0 + j], 0, 0, 0);
+            }
         }
     }
     l = quad_rows_sum(l);
@@ -180,6 +200,29 @@ latent_attention_mfma_kernel(bf16_t *__restrict__ out, float *__restrict__ part_
         w.h[2] = float_to_bf16_bits(o[dt][2] * mul); w.h[3] = float_to_bf16_bits(o[dt][3] * mul);
         *reinterpret_cast<uint2 *>(orow + 16 * dt) = w.u2;
     }
+}
+
+#define LAT_KERNEL_ARGS                                                                                        \
+    bf16_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_ml, const bf16_t *__restrict__ q, \
+        const bf16_t *__restrict__ cache, const bf16_t *__restrict__ cache_t, const int *__restrict__ block_table, \
+        int max_blocks, const int *__restrict__ item_entry, const int *__restrict__ item_row0,                \
+        const int *__restrict__ entry_seat, const int *__restrict__ entry_q_start,                            \
+        const int *__restrict__ entry_start_pos, int heads, int page_size, float scale, int window,           \
+        int keep_first, const float *__restrict__ sinks, int splits, int per_split
+#define LAT_KERNEL_PASS                                                                                        \
+    out, part_o, part_ml, q, cache, cache_t, block_table, max_blocks, item_entry, item_row0, entry_seat,       \
+        entry_q_start, entry_start_pos, heads, page_size, scale, window, keep_first, sinks, splits, per_split
+
+template <int NDT, int NKS>
+__global__ void __launch_bounds__(KVA_WAVE) latent_attention_mfma_kernel(LAT_KERNEL_ARGS) {
+    latent_attention_mfma_body<NDT, NKS>(LAT_KERNEL_PASS);
+}
+
+// large rows: one wavefront a SIMD, so that a block's keys (2 NKS fragments) fit the registers beside the result
+template <int NDT, int NKS>
+__global__ void __launch_bounds__(KVA_WAVE) __attribute__((amdgpu_waves_per_eu(1, 1)))
+latent_attention_mfma_wide_kernel(LAT_KERNEL_ARGS) {
+    latent_attention_mfma_body<NDT, NKS>(LAT_KERNEL_PASS);
 }
 
 // out[row] = sum_s w_s o_s / (sum_s w_s l_s + exp(sink)), w_s = exp2(m_s - max); one workgroup a row
@@ -230,7 +273,9 @@ extern "C" int kva_latent_attention_mfma(void *out, float *part_o, float *part_m
     bool done = false;
 #define LAUNCH_ONE(NDT, NKS)                                                                                   \
     if (!done && rank == NDT * 16 && key_dim == NKS * 32) {                                                    \
-        hipLaunchKernelGGL((latent_attention_mfma_kernel<NDT, NKS>), grid, block, 0, stream, (bf16_t *)out,    \
+        auto kernel = (4 * NDT + 8 * NKS > 160) ? latent_attention_mfma_wide_kernel<NDT, NKS>                  \
+                                                : latent_attention_mfma_kernel<NDT, NKS>;                      \
+        hipLaunchKernelGGL(kernel, grid, block, 0, stream, (bf16_t *)out,                                      \
                            part_o, part_ml, (const bf16_t *)q, (const bf16_t *)cache, (const bf16_t *)cache_t, \
                            block_table, max_blocks, item_entry, item_row0, entry_seat, entry_q_start,          \
                            entry_start_pos, heads, page_size, scale, window, keep_first, sinks, splits,        \
@@ -322,13 +367,12 @@ gqa_attention_rows_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, 
             // K pages are [D / 8][page_size][8]: chunk 4 ks + g of key `key`
             const bf16_t *kp = k_cache + ((size_t)page[t] * kv_heads + kvh) * page_size * D +
                                ((size_t)g * page_size + key % page_size) * 8;
+            Frag8 kf[NKS];
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks) kf[ks].u4 = *reinterpret_cast<const uint4 *>(kp + (size_t)ks * 4 * page_size * 8);
             s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int ks = 0; ks < NKS; ++ks) {
-                Frag8 kf;
-                kf.u4 = *reinterpret_cast<const uint4 *>(kp + (size_t)ks * 4 * page_size * 8);
-                s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[ks].v, s[t], 0, 0, 0);
-            }
+            for (int ks = 0; ks < NKS; ++ks) s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[ks].v, qf[ks].v, s[t], 0, 0, 0);
         }
         float sv[8], mx = -INFINITY;
 #pragma unroll
@@ -372,14 +416,22 @@ gqa_attention_rows_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, 
             }
             vrow[t] = v_cache + (((size_t)page[t] * kv_heads + kvh) * DV + r) * page_size + key0 % page_size;
         }
+        constexpr int VC = NDT < 8 ? NDT : 8;                          // value tiles asked for together
 #pragma unroll
-        for (int dt = 0; dt < NDT; ++dt) {
-            Frag8 vv;
-            vv.u2[0] = *reinterpret_cast<const uint2 *>(vrow[0] + (size_t)dt * 16 * page_size);
-            vv.u2[1] = *reinterpret_cast<const uint2 *>(vrow[1] + (size_t)dt * 16 * page_size);
-            vv.u2[0].x &= keep[0].x; vv.u2[0].y &= keep[0].y;
-            vv.u2[1].x &= keep[1].x; vv.u2[1].y &= keep[1].y;
-            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv.v, pf.v, o[dt], 0, 0, 0);
+        for (int d0 = 0; d0 < NDT; d0 += VC) {
+            Frag8 vv[VC];
+#pragma unroll
+            for (int j = 0; j < VC; ++j) {
+                vv[j].u2[0] = *reinterpret_cast<const uint2 *>(vrow[0] + (size_t)(d0 + j) * 16 * page_size);
+                vv[j].u2[1] = *reinterpret_cast<const uint2 *>(vrow[1] + (size_t)(d0 + j) * 16 * page_size);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < VC; ++j) {
+                vv[j].u2[0].x &= keep[0].x; vv[j].u2[0].y &= keep[0].y;
+                vv[j].u2[1].x &= keep[1].x; vv[j].u2[1].y &= keep[1].y;
+                o[d0 + j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv[j].v, pf.v, o[d0 + j], 0, 0, 0);
+            }
         }
     }
     l = quad_rows_sum(l);

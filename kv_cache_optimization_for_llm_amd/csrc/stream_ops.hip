@@ -115,10 +115,34 @@ __global__ void act_mul_kernel(void *__restrict__ out, const void *__restrict__ 
     st_from_float(out, dtype, t * inter + i, kva_activate(g, act) * u);
 }
 
+// bf16, inter a multiple of 8: a thread takes 8 neighbouring columns with 16-byte loads and stores
+__global__ void act_mul_vec_kernel(uint4 *__restrict__ out, const uint4 *__restrict__ gu, int inter8, int act) {
+    const size_t t = blockIdx.y;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= inter8) return;
+    const uint4 gv = gu[t * 2 * inter8 + i], uv = gu[t * 2 * inter8 + inter8 + i];
+    const uint32_t gw[4] = {gv.x, gv.y, gv.z, gv.w}, uw[4] = {uv.x, uv.y, uv.z, uv.w};
+    uint32_t ow[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float g0 = bf16_bits_to_float((uint16_t)(gw[j] & 0xffffu)), g1 = bf16_bits_to_float((uint16_t)(gw[j] >> 16));
+        const float u0 = bf16_bits_to_float((uint16_t)(uw[j] & 0xffffu)), u1 = bf16_bits_to_float((uint16_t)(uw[j] >> 16));
+        ow[j] = (uint32_t)float_to_bf16_bits(kva_activate(g0, act) * u0) |
+                ((uint32_t)float_to_bf16_bits(kva_activate(g1, act) * u1) << 16);
+    }
+    out[t * inter8 + i] = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+}
+
 extern "C" int kva_act_mul(void *out, const void *gate_up, int rows, int inter, int act, int dtype, hipStream_t stream) {
     KVA_REQUIRE(rows >= 0 && rows <= 65535 && inter > 0, "act_mul: bad sizes");
     KVA_REQUIRE(act >= KVA_ACT_SILU && act <= KVA_ACT_GELU_TANH, "act_mul: unknown activation %d", act);
     if (rows == 0) return KVA_OK;
+    if (dtype == KVA_BF16 && inter % 8 == 0) {
+        hipLaunchKernelGGL(act_mul_vec_kernel, dim3((inter / 8 + 255) / 256, rows), dim3(256), 0, stream, (uint4 *)out,
+                           (const uint4 *)gate_up, inter / 8, act);
+        KVA_CHECK_LAUNCH("act_mul");
+        return KVA_OK;
+    }
     hipLaunchKernelGGL(act_mul_kernel, dim3((inter + 255) / 256, rows), dim3(256), 0, stream, out, gate_up, dtype,
                        inter, act);
     KVA_CHECK_LAUNCH("act_mul");

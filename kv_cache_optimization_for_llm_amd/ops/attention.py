@@ -381,8 +381,9 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
                 and K.attention_rows_mfma_supported(head_dim, value_dim, kv.page_size):
             from .latent_attention import choose_ranges
             item_entry, item_row0, _ = batch.attention_items(num_q_heads // num_kv_heads, 1, "all")
-            # a window bounds what a row reads whatever the context: its keys are not cut into ranges
-            ranges, per = (1, 0) if window > 0 else choose_ranges(item_entry.shape[0] * num_kv_heads, batch.max_context)
+            # (with a window most ranges of a long context hold no visible key: their wavefronts end at once)
+            ranges, per = choose_ranges(item_entry.shape[0] * num_kv_heads, batch.max_context,
+                                        window + keep_first if window > 0 else 0)
             return K.attention_rows_mfma(qkv, qkv.shape[1], out, kv.k_cache, kv.v_cache, kv.block_table, item_entry,
                                          item_row0, batch.entry_seat, batch.entry_q_start, batch.entry_start_pos,
                                          num_q_heads, num_kv_heads, head_dim, scale, window, keep_first, sinks,

@@ -667,6 +667,12 @@ def heads_matmul(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.T
     orr, oh = (out.stride(0), out.stride(1)) if rows > 1 else (max(out.stride(0), (heads - 1) * out.stride(1) + n), out.stride(1))
     if heads == 1:
         xh, oh = max(xh, k), max(oh, n)
+    if x.dtype == torch.bfloat16 and x.data_ptr() % 16 == 0 and out.data_ptr() % 8 == 0 \
+            and hip_lib().kva_heads_matmul_mfma_supported(k, xr, xh):
+        # bf16 with a K that has an instance: the matrix cores
+        check(hip_lib().kva_heads_matmul_mfma(_dev(out, "out", contiguous=False), orr, oh, _dev(x, "x", contiguous=False),
+                                              xr, xh, _dev(w, "w"), rows, heads, n, k, _stream()), "heads_matmul_mfma")
+        return out
     check(hip_lib().kva_heads_matmul(_dev(out, "out", contiguous=False), orr, oh, _dev(x, "x", contiguous=False), xr, xh,
                                      _dev(w, "w"), rows, heads, n, k, dtype_code(x.dtype), _stream()), "heads_matmul")
     return out

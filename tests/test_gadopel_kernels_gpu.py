@@ -240,10 +240,14 @@ def test_low_rank_entry_is_normed_rotated_and_cached(dtype, gpu):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("rows, heads, n, k", [(1, 3, 40, 16), (9, 5, 24, 8), (130, 2, 70, 96), (3, 1, 8, 200)])
-def test_per_head_products_into_column_ranges(rows, heads, n, k, dtype, gpu):
-    x_wide = rnd((rows, heads, k + 5), 1, DT[dtype]).to(gpu)
-    out_wide = torch.zeros((rows, heads, n + 3), dtype=DT[dtype], device=gpu)
+@pytest.mark.parametrize("x_pad, out_pad", [(5, 3), (8, 4), (0, 0)])
+@pytest.mark.parametrize("rows, heads, n, k", [(1, 3, 40, 16), (9, 5, 24, 8), (130, 2, 70, 96), (3, 1, 8, 200),
+                                               (1, 16, 512, 128), (40, 3, 128, 512), (300, 4, 48, 64)])
+def test_per_head_products_into_column_ranges(rows, heads, n, k, x_pad, out_pad, dtype, gpu):
+    """(bf16 rows whose strides are multiples of 8 and whose K has an instance take the matrix
+    cores, everything else the plain kernel: both against the same sums)"""
+    x_wide = rnd((rows, heads, k + x_pad), 1, DT[dtype]).to(gpu)
+    out_wide = torch.zeros((rows, heads, n + out_pad), dtype=DT[dtype], device=gpu)
     w = rnd((heads, n, k), 2, DT[dtype], 0.3).to(gpu)
     lat_ops.heads_product(x_wide[:, :, :k], w, out_wide[:, :, :n])
     want = torch.einsum("thk,hnk->thn", x_wide[:, :, :k].double(), w.double())
