@@ -97,6 +97,75 @@ qk_encode_cache_kernel(T *__restrict__ qkv, int row_stride, int k_off, int v_off
     }
 }
 
+// bf16, interleaved pairs, heads of 8 * 2^k elements (up to 512): a lane takes 8 neighbouring
+// elements of a head (four whole pairs: 16 bytes in, 16 bytes out - one chunk of the K page), the
+// 2^k lanes of a head add their squares up between them.
+__global__ void __launch_bounds__(256)
+qk_encode_cache_vec_kernel(bf16_t *__restrict__ qkv, int row_stride, int k_off, int v_off, bf16_t *__restrict__ k_cache,
+                           bf16_t *__restrict__ v_cache, const float *__restrict__ cos_table,
+                           const float *__restrict__ sin_table, const int *__restrict__ positions,
+                           const int *__restrict__ slot_mapping, int num_q_heads, int num_kv_heads, int head_dim,
+                           int value_dim, int rot, float unit_eps, int page_size) {
+    const int t = blockIdx.x;
+    bf16_t *row = qkv + (size_t)t * row_stride;
+    const int pos = positions[t];
+    const int half = rot / 2, vecs = head_dim / 8;                // lanes a head
+    const float *cs = cos_table + (size_t)pos * half, *sn = sin_table + (size_t)pos * half;
+    const int slot = slot_mapping ? slot_mapping[t] : -1;
+    const int page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
+    const int total = (num_q_heads + num_kv_heads) * vecs;
+    for (int w0 = 0; w0 < total; w0 += blockDim.x) {              // (uniform trip count: the lanes of a head shuffle)
+        const int w = w0 + threadIdx.x;
+        const bool on = w < total;
+        const int head = on ? w / vecs : 0, j = on ? w % vecs : 0;
+        const bool is_q = head < num_q_heads;
+        bf16_t *h = is_q ? row + (size_t)head * head_dim : row + k_off + (size_t)(head - num_q_heads) * head_dim;
+        float x[8], y[8];
+        const uint4 in = *reinterpret_cast<const uint4 *>(h + 8 * j);
+        const uint32_t iw[4] = {in.x, in.y, in.z, in.w};
+        float sq = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            x[2 * i] = bf16_bits_to_float((uint16_t)(iw[i] & 0xffffu));
+            x[2 * i + 1] = bf16_bits_to_float((uint16_t)(iw[i] >> 16));
+            const int p = 4 * j + i;                              // pair (2p, 2p + 1) of the head
+            if (p < half) {
+                const float co = cs[p], si = sn[p];
+                y[2 * i] = x[2 * i] * co - x[2 * i + 1] * si;
+                y[2 * i + 1] = x[2 * i + 1] * co + x[2 * i] * si;
+            } else {
+                y[2 * i] = x[2 * i];
+                y[2 * i + 1] = x[2 * i + 1];
+            }
+            sq += y[2 * i] * y[2 * i] + y[2 * i + 1] * y[2 * i + 1];
+        }
+        float mul = 1.f;
+        if (unit_eps >= 0.f) {
+            for (int o = vecs / 2; o > 0; o >>= 1) sq += __shfl_xor(sq, o, KVA_WAVE);
+            mul = 1.0f / sqrtf(sq / (float)head_dim + unit_eps);
+        }
+        uint32_t ow[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            ow[i] = (uint32_t)float_to_bf16_bits(y[2 * i] * mul) | ((uint32_t)float_to_bf16_bits(y[2 * i + 1] * mul) << 16);
+        const uint4 res = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+        if (!on) continue;
+        if (is_q) {
+            *reinterpret_cast<uint4 *>(h + 8 * j) = res;
+        } else if (slot >= 0) {
+            bf16_t *kdst = k_cache + ((size_t)page * num_kv_heads + (head - num_q_heads)) * page_size * head_dim;
+            *reinterpret_cast<uint4 *>(kdst + kva_k_at(off, 8 * j, page_size, 8)) = res;
+        }
+    }
+    if (slot >= 0) {
+        const bf16_t *v = row + v_off;
+        for (int w = threadIdx.x; w < num_kv_heads * value_dim; w += blockDim.x) {
+            const int kvh = w / value_dim, j = w % value_dim;
+            v_cache[(((size_t)page * num_kv_heads + kvh) * value_dim + j) * page_size + off] = v[w];
+        }
+    }
+}
+
 extern "C" int kva_qk_encode_cache(void *qkv, int row_stride, int k_off, int v_off, void *k_cache, void *v_cache,
                                    const float *cos_table, const float *sin_table, const int *positions,
                                    const int *slot_mapping, int tokens, int num_q_heads, int num_kv_heads,
@@ -115,6 +184,15 @@ extern "C" int kva_qk_encode_cache(void *qkv, int row_stride, int k_off, int v_o
                 "qk_encode_cache: the row layout [q | k | v] does not fit its stride");
     if (tokens == 0) return KVA_OK;
     if (rot == 0) cos_table = sin_table = reinterpret_cast<const float *>(qkv);     // never read
+    const int vecs = head_dim / 8;
+    if (dtype == KVA_BF16 && interleaved && head_dim % 8 == 0 && (vecs & (vecs - 1)) == 0 && vecs <= KVA_WAVE &&
+        row_stride % 8 == 0 && k_off % 8 == 0 && (reinterpret_cast<uintptr_t>(qkv) & 15) == 0) {
+        hipLaunchKernelGGL(qk_encode_cache_vec_kernel, dim3(tokens), dim3(256), 0, stream, (bf16_t *)qkv, row_stride,
+                           k_off, v_off, (bf16_t *)k_cache, (bf16_t *)v_cache, cos_table, sin_table, positions,
+                           slot_mapping, num_q_heads, num_kv_heads, head_dim, value_dim, rot, unit_eps, page_size);
+        KVA_CHECK_LAUNCH("qk_encode_cache");
+        return KVA_OK;
+    }
     if (dtype == KVA_F32)
         hipLaunchKernelGGL(qk_encode_cache_kernel<float>, dim3(tokens), dim3(256), 0, stream, (float *)qkv, row_stride,
                            k_off, v_off, (float *)k_cache, (float *)v_cache, cos_table, sin_table, positions,

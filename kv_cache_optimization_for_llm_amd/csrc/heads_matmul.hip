@@ -14,7 +14,7 @@
 template <typename T>
 __global__ void __launch_bounds__(256)
 heads_matmul_kernel(T *__restrict__ out, int o_row, int o_head, const T *__restrict__ x, int x_row, int x_head,
-                    const T *__restrict__ w, int M, int N, int K) {
+                    const T *__restrict__ w, int M, int N, int K, const T *__restrict__ gate, int g_row) {
     __shared__ float Xs[HM_BK][HM_BM + 4];
     __shared__ float Ws[HM_BK][HM_BN + 4];
     const int h = blockIdx.z;
@@ -59,16 +59,19 @@ heads_matmul_kernel(T *__restrict__ out, int o_row, int o_head, const T *__restr
     for (int i = 0; i < 4; ++i) {
         const int m = m0 + ty * 4 + i;
         if (m >= M) continue;
+        // (optional) the head's gate: the row's outputs of head h times sigmoid(gate[m, h])
+        const float gmul = gate ? 1.0f / (1.0f + expf(-to_float(gate[(size_t)m * g_row + h]))) : 1.0f;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int n = n0 + tx * 4 + j;
-            if (n < N) out[(size_t)m * o_row + (size_t)h * o_head + n] = from_float<T>(acc[i][j]);
+            if (n < N) out[(size_t)m * o_row + (size_t)h * o_head + n] = from_float<T>(acc[i][j] * gmul);
         }
     }
 }
 
 extern "C" int kva_heads_matmul(void *out, int o_row, int o_head, const void *x, int x_row, int x_head,
-                                const void *w, int rows, int heads, int N, int K, int dtype, hipStream_t stream) {
+                                const void *w, int rows, int heads, int N, int K, const void *gate, int g_row,
+                                int dtype, hipStream_t stream) {
     KVA_REQUIRE(rows >= 0 && heads > 0 && heads <= 65535 && N > 0 && K > 0, "heads_matmul: bad sizes");
     KVA_REQUIRE(x_head >= K && o_head >= N && x_row >= (heads - 1) * x_head + K && o_row >= (heads - 1) * o_head + N,
                 "heads_matmul: strides do not fit %d heads of %d -> %d", heads, K, N);
@@ -77,10 +80,10 @@ extern "C" int kva_heads_matmul(void *out, int o_row, int o_head, const void *x,
     KVA_REQUIRE(grid.y <= 65535, "heads_matmul: %d rows are too many for one launch", rows);
     if (dtype == KVA_F32)
         hipLaunchKernelGGL(heads_matmul_kernel<float>, grid, block, 0, stream, (float *)out, o_row, o_head,
-                           (const float *)x, x_row, x_head, (const float *)w, rows, N, K);
+                           (const float *)x, x_row, x_head, (const float *)w, rows, N, K, (const float *)gate, g_row);
     else if (dtype == KVA_BF16)
         hipLaunchKernelGGL(heads_matmul_kernel<bf16_t>, grid, block, 0, stream, (bf16_t *)out, o_row, o_head,
-                           (const bf16_t *)x, x_row, x_head, (const bf16_t *)w, rows, N, K);
+                           (const bf16_t *)x, x_row, x_head, (const bf16_t *)w, rows, N, K, (const bf16_t *)gate, g_row);
     else KVA_REQUIRE(false, "heads_matmul: unsupported dtype %d", dtype);
     KVA_CHECK_LAUNCH("heads_matmul");
     return KVA_OK;
@@ -97,7 +100,8 @@ extern "C" int kva_heads_matmul(void *out, int o_row, int o_head, const void *x,
 template <int NKS>
 __global__ void __launch_bounds__(KVA_WAVE)
 heads_matmul_mfma_kernel(bf16_t *__restrict__ out, int o_row, int o_head, const bf16_t *__restrict__ x, int x_row,
-                         int x_head, const bf16_t *__restrict__ w, int M, int N, int tiles_per_wave) {
+                         int x_head, const bf16_t *__restrict__ w, int M, int N, int tiles_per_wave,
+                         const bf16_t *__restrict__ gate, int g_row) {
     constexpr int K = NKS * 32;
     const int lane = threadIdx.x, r = lane & 15, g = lane >> 4;
     const int n0 = blockIdx.x * 16, h = blockIdx.y;
@@ -120,6 +124,10 @@ heads_matmul_mfma_kernel(bf16_t *__restrict__ out, int o_row, int o_head, const 
             acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[ks].v, xf.v, acc, 0, 0, 0);
         }
         // lane (row t = r, group g) holds outputs n0 + 4 g .. + 3 of its row
+        if (gate) {
+            const float gmul = 1.0f / (1.0f + expf(-to_float(gate[(size_t)t * g_row + h])));
+            acc[0] *= gmul; acc[1] *= gmul; acc[2] *= gmul; acc[3] *= gmul;
+        }
         if (tile * 16 + r < M) {
             bf16_t *o = out + (size_t)t * o_row + (size_t)h * o_head + n0 + 4 * g;
             if (n0 + 4 * g + 3 < N && ((o_row | o_head) % 4 == 0)) {
@@ -147,7 +155,8 @@ extern "C" int kva_heads_matmul_mfma_supported(int K, int x_row, int x_head) {
 }
 
 extern "C" int kva_heads_matmul_mfma(void *out, int o_row, int o_head, const void *x, int x_row, int x_head,
-                                     const void *w, int rows, int heads, int N, int K, hipStream_t stream) {
+                                     const void *w, int rows, int heads, int N, int K, const void *gate, int g_row,
+                                     hipStream_t stream) {
     KVA_REQUIRE(rows >= 0 && heads > 0 && heads <= 65535 && N > 0, "heads_matmul_mfma: bad sizes");
     KVA_REQUIRE(kva_heads_matmul_mfma_supported(K, x_row, x_head),
                 "heads_matmul_mfma: no instance for K = %d with strides %d / %d", K, x_row, x_head);
@@ -164,7 +173,8 @@ extern "C" int kva_heads_matmul_mfma(void *out, int o_row, int o_head, const voi
 #define LAUNCH_ONE(NKS)                                                                                          \
     if (!done && K == NKS * 32) {                                                                                \
         hipLaunchKernelGGL(heads_matmul_mfma_kernel<NKS>, grid, block, 0, stream, (bf16_t *)out, o_row, o_head,  \
-                           (const bf16_t *)x, x_row, x_head, (const bf16_t *)w, rows, N, per_wave);              \
+                           (const bf16_t *)x, x_row, x_head, (const bf16_t *)w, rows, N, per_wave,               \
+                           (const bf16_t *)gate, g_row);                                                         \
         done = true;                                                                                             \
     }
     HM_INSTANCES(LAUNCH_ONE)

@@ -655,11 +655,18 @@ def latent_encode_cache(y: torch.Tensor, kv_off: int, q_lat: torch.Tensor, cache
         1 if interleaved else 0, dtype_code(y.dtype), _stream()), "latent_encode_cache")
 
 
-def heads_matmul(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+def heads_matmul(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gates: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``out[t, h, :] = w[h] @ x[t, h, :]`` for ``w`` ``[heads, N, K]``.  ``x`` ``[T, heads, K]`` and
-    ``out`` ``[T, heads, N]`` may be views into wider buffers (unit stride along the last axis)."""
+    ``out`` ``[T, heads, N]`` may be views into wider buffers (unit stride along the last axis).
+    With ``gates`` (``[T, heads]``, a column range of another buffer) head h of row t is multiplied
+    by ``sigmoid(gates[t, h])``."""
     heads, n, k = w.shape
     rows = x.shape[0]
+    g_row = 0
+    if gates is not None:
+        if gates.shape != (rows, heads) or gates.dtype != x.dtype or gates.stride(1) != 1:
+            raise KernelError(f"heads_matmul: gates {tuple(gates.shape)} do not fit {rows} rows of {heads} heads")
+        g_row = gates.stride(0) if rows > 1 else heads
     if x.shape != (rows, heads, k) or out.shape != (rows, heads, n) or x.stride(2) != 1 or out.stride(2) != 1 \
             or not (x.dtype == w.dtype == out.dtype):
         raise KernelError(f"heads_matmul: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
@@ -671,10 +678,14 @@ def heads_matmul(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.T
             and hip_lib().kva_heads_matmul_mfma_supported(k, xr, xh):
         # bf16 with a K that has an instance: the matrix cores
         check(hip_lib().kva_heads_matmul_mfma(_dev(out, "out", contiguous=False), orr, oh, _dev(x, "x", contiguous=False),
-                                              xr, xh, _dev(w, "w"), rows, heads, n, k, _stream()), "heads_matmul_mfma")
+                                              xr, xh, _dev(w, "w"), rows, heads, n, k,
+                                              None if gates is None else _dev(gates, "gates", contiguous=False), g_row,
+                                              _stream()), "heads_matmul_mfma")
         return out
     check(hip_lib().kva_heads_matmul(_dev(out, "out", contiguous=False), orr, oh, _dev(x, "x", contiguous=False), xr, xh,
-                                     _dev(w, "w"), rows, heads, n, k, dtype_code(x.dtype), _stream()), "heads_matmul")
+                                     _dev(w, "w"), rows, heads, n, k,
+                                     None if gates is None else _dev(gates, "gates", contiguous=False), g_row,
+                                     dtype_code(x.dtype), _stream()), "heads_matmul")
     return out
 
 

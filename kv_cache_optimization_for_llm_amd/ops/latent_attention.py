@@ -6,10 +6,10 @@ import torch
 from . import kernels as K
 
 
-def heads_product(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+def heads_product(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gates=None) -> torch.Tensor:
     """``out[t, h] = w[h] @ x[t, h]`` for ``w`` ``[heads, N, K]``; ``x`` and ``out`` may be views into
-    wider buffers."""
-    return K.heads_matmul(x, w, out)
+    wider buffers.  ``gates`` ``[T, heads]``: head h of row t times ``sigmoid(gates[t, h])``."""
+    return K.heads_matmul(x, w, out, gates)
 
 
 TRANSPOSED = "latent_t"         # name of the cache array that holds the latent part a second time, [rank, page_size]

@@ -55,9 +55,9 @@ _HIP_SIGNATURES = {
     "kva_attention_rows_mfma_supported": [I, I, I],
     "kva_attention_rows_mfma": [P, P, P, P, I, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P, I, I, P],
     "kva_latent_attention_mfma": [P, P, P, P, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P, I, I, P],
-    "kva_heads_matmul": [P, I, I, P, I, I, P, I, I, I, I, I, P],
+    "kva_heads_matmul": [P, I, I, P, I, I, P, I, I, I, I, P, I, I, P],
     "kva_heads_matmul_mfma_supported": [I, I, I],
-    "kva_heads_matmul_mfma": [P, I, I, P, I, I, P, I, I, I, I, P],
+    "kva_heads_matmul_mfma": [P, I, I, P, I, I, P, I, I, I, I, P, I, P],
     "kva_attention_mfma": [P, P, P, P, I, P, P, P, I, P, P, P, I, I, P, P, P, I, I, I, I, I, F, I, I, I, I, I, I, I, P],
     "kva_attention_mfma_rope": [P, P, P, P, I, P, P, P, I, P, I, I, I, I, I, I, F, I, I, I, I, P, P, P, I, P],
     "kva_attention_mfma_rope_supported": [I, I, I],

@@ -142,7 +142,7 @@ class LatentAttention(Mixer):
         o_lat = torch.empty((T, H, self.rank), dtype=x.dtype, device=x.device)
         lat_ops.latent_attention(q_lat, o_lat, kv, batch, self.scale, self.window, self.keep_first, self.sinks)
         out = torch.empty((T, H * self.value_dim), dtype=x.dtype, device=x.device)
-        lat_ops.heads_product(o_lat, self.up_v, out.view(T, H, self.value_dim))
-        if self.has_gate:
-            K.head_gate(out, y[:, self.gate_off:self.gate_off + H], H)
+        # the value expansion behind the attention, the head's output gate in the same pass
+        lat_ops.heads_product(o_lat, self.up_v, out.view(T, H, self.value_dim),
+                              gates=y[:, self.gate_off:self.gate_off + H] if self.has_gate else None)
         return self.o(out)

@@ -253,6 +253,13 @@ def test_per_head_products_into_column_ranges(rows, heads, n, k, x_pad, out_pad,
     want = torch.einsum("thk,hnk->thn", x_wide[:, :, :k].double(), w.double())
     close(out_wide[:, :, :n], want, TOL[dtype], "per-head product")
     assert (out_wide[:, :, n:] == 0).all()
+    # with a gate per head, read from a column range of a wider buffer
+    wide = rnd((rows, heads + 6), 3, DT[dtype]).to(gpu)
+    lat_ops.heads_product(x_wide[:, :, :k], w, out_wide[:, :, :n], gates=wide[:, 2:2 + heads])
+    close(out_wide[:, :, :n], want * torch.sigmoid(wide[:, 2:2 + heads].double())[:, :, None], TOL[dtype], "gated")
+    got = wide[:, 2:2 + heads].clone()
+    K.head_gate(got_x := torch.ones((rows, heads * 4), dtype=DT[dtype], device=gpu), wide[:, 2:2 + heads], heads)
+    close(got_x.view(rows, heads, 4)[:, :, 0], torch.sigmoid(got.double()), TOL[dtype], "the gate alone")
 
 
 @pytest.mark.parametrize("per_range", [0, 32, 96])
