@@ -52,6 +52,7 @@ latent_attention_mfma_body(bf16_t *__restrict__ out, float *__restrict__ part_o,
     const int my_pos = start_pos + my_row / heads;
     const int my_lo = (window > 0 && my_pos - window + 1 > 0) ? my_pos - window + 1 : 0;
     const int item_lo = (window > 0 && pos_lo - window + 1 > 0) ? pos_lo - window + 1 : 0;
+    const int hi_lo = (window > 0 && item_hi - window + 1 > 0) ? item_hi - window + 1 : 0;     // where the last row's window starts
     const size_t my_global = (size_t)q_start * heads + my_row;      // row of q / out
 
     // Q^T in operand layout: lane (row r, group g) holds elements 32 ks + 8 g .. + 7 of its row;
@@ -107,27 +108,37 @@ latent_attention_mfma_body(bf16_t *__restrict__ out, float *__restrict__ part_o,
             }
         }
         // mask and online softmax: lane (row r, group g) holds keys kstart + 16 t + 4 g + i
+        // a block that every row of the item sees whole (the common one) needs no mask: wave-uniform
+        const bool whole = mapped[0] && mapped[1] && kstart >= k_begin && kstart + 32 <= k_end && kstart + 31 <= pos_lo &&
+                           (kstart >= hi_lo || kstart + 32 <= keep_first);
         float sv[8], mx = -INFINITY;
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const int key = kstart + 16 * t + 4 * g + i;
-                const bool vis = row_valid && mapped[t] && key <= my_pos && (key >= my_lo || key < keep_first) &&
-                                 key >= k_begin && key < k_end;
-                const float x = vis ? s[t][i] * scale2 : -INFINITY;
+                float x = s[t][i] * scale2;
+                if (!whole) {
+                    const int key = kstart + 16 * t + 4 * g + i;
+                    const bool vis = row_valid && mapped[t] && key <= my_pos && (key >= my_lo || key < keep_first) &&
+                                     key >= k_begin && key < k_end;
+                    x = vis ? x : -INFINITY;
+                }
                 sv[t * 4 + i] = x;
                 mx = fmaxf(mx, x);
             }
-        const float m_new = fmaxf(m, quad_rows_max(mx));
-        const float ref = (m_new == -INFINITY) ? 0.f : m_new;
-        const float corr = __builtin_amdgcn_exp2f(m - ref);           // exp2(-inf) = 0
-        l *= corr;
+        // the running maximum moves in few blocks: only then are l and O re-based (wave-uniform branch)
+        const float bm = quad_rows_max(mx);
+        if (__builtin_amdgcn_ballot_w64(bm > m) != 0) {
+            const float m_new = fmaxf(m, bm);
+            const float corr = __builtin_amdgcn_exp2f(m - ((m_new == -INFINITY) ? 0.f : m_new));     // exp2(-inf) = 0
+            l *= corr;
 #pragma unroll
-        for (int dt = 0; dt < NDT; ++dt) {
-            o[dt][0] *= corr; o[dt][1] *= corr; o[dt][2] *= corr; o[dt][3] *= corr;
+            for (int dt = 0; dt < NDT; ++dt) {
+                o[dt][0] *= corr; o[dt][1] *= corr; o[dt][2] *= corr; o[dt][3] *= corr;
+            }
+            m = m_new;
         }
-        m = m_new;
+        const float ref = (m == -INFINITY) ? 0.f : m;
         Frag8 pf;
 #pragma unroll
         for (int j = 0; j < 8; j += 2) {
@@ -301,7 +312,7 @@ extern "C" int kva_latent_attention_mfma(void *out, float *part_o, float *part_m
 // positions visible, a sink per head, values of another size than the keys.  Rows of a tile are
 // (token, query head of the kv head's group) pairs, row = token_in_entry * G + head_in_group; one
 // wavefront per (item, kv head, key range).  D = 32 NKS key elements, DV = 16 NDT value elements.
-template <int NDT, int NKS>
+template <int NDT, int NKS, int RT>
 __global__ void __launch_bounds__(KVA_WAVE)
 gqa_attention_rows_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_ml,
                           const bf16_t *__restrict__ q, int q_stride, const bf16_t *__restrict__ k_cache,
@@ -311,6 +322,8 @@ gqa_attention_rows_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, 
                           const int *__restrict__ entry_start_pos, int heads, int kv_heads, int page_size,
                           float scale, int window, int keep_first, const float *__restrict__ sinks, int splits,
                           int per_split) {
+    // RT tiles of 16 rows share every key and value fragment the wavefront loads (prompt portions:
+    // half the loads a product with RT = 2)
     constexpr int DV = NDT * 16, D = NKS * 32;
     const int lane = threadIdx.x, r = lane & 15, g = lane >> 4;
     const int item = blockIdx.x, kvh = blockIdx.y / splits, split = blockIdx.y % splits;
@@ -321,27 +334,33 @@ gqa_attention_rows_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, 
     const int *bt = block_table + (size_t)entry_seat[e] * max_blocks;
     const int rows = q_len * group;
     if (row0 >= rows) return;
-    const int last_row = min(row0 + 15, rows - 1);
+    const int last_row = min(row0 + 16 * RT - 1, rows - 1);
     const int item_hi = start_pos + last_row / group;
     const int pos_lo = start_pos + row0 / group;
-    const int my_row = min(row0 + r, rows - 1);
-    const bool row_valid = row0 + r < rows;
-    const int my_pos = start_pos + my_row / group;
-    const int my_head = kvh * group + my_row % group;
-    const int my_lo = (window > 0 && my_pos - window + 1 > 0) ? my_pos - window + 1 : 0;
     const int item_lo = (window > 0 && pos_lo - window + 1 > 0) ? pos_lo - window + 1 : 0;
-    const size_t my_token = (size_t)q_start + my_row / group;
-
-    Frag8 qf[NKS];
-    {
-        const bf16_t *qrow = q + my_token * q_stride + (size_t)my_head * D + 8 * g;
+    const int hi_lo = (window > 0 && item_hi - window + 1 > 0) ? item_hi - window + 1 : 0;     // where the last row's window starts
+    int my_pos[RT], my_lo[RT], my_head[RT];
+    bool row_valid[RT];
+    size_t my_token[RT];
+    Frag8 qf[RT][NKS];
+    f32x4 o[RT][NDT];
+    float m[RT], l[RT];
 #pragma unroll
-        for (int ks = 0; ks < NKS; ++ks) qf[ks].u4 = *reinterpret_cast<const uint4 *>(qrow + 32 * ks);
+    for (int rt = 0; rt < RT; ++rt) {
+        const int row = min(row0 + 16 * rt + r, rows - 1);
+        row_valid[rt] = row0 + 16 * rt + r < rows;
+        my_pos[rt] = start_pos + row / group;
+        my_head[rt] = kvh * group + row % group;
+        my_lo[rt] = (window > 0 && my_pos[rt] - window + 1 > 0) ? my_pos[rt] - window + 1 : 0;
+        my_token[rt] = (size_t)q_start + row / group;
+        const bf16_t *qrow = q + my_token[rt] * q_stride + (size_t)my_head[rt] * D + 8 * g;
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) qf[rt][ks].u4 = *reinterpret_cast<const uint4 *>(qrow + 32 * ks);
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt) o[rt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        m[rt] = -INFINITY;
+        l[rt] = 0.f;
     }
-    f32x4 o[NDT];
-#pragma unroll
-    for (int dt = 0; dt < NDT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-    float m = -INFINITY, l = 0.f;
     const float scale2 = scale * LAT_LOG2E;
 
     int k_begin = 0, k_end = item_hi + 1;
@@ -360,52 +379,18 @@ gqa_attention_rows_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, 
             mapped[t] = p >= 0;
             page[t] = p >= 0 ? p : 0;
         }
-        f32x4 s[2];
+        // every load of the block is asked for before the first product
+        Frag8 kf[2][NKS], vv[NDT];
+        uint2 keep[2];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             const int key = kstart + 16 * t + r;
             // K pages are [D / 8][page_size][8]: chunk 4 ks + g of key `key`
             const bf16_t *kp = k_cache + ((size_t)page[t] * kv_heads + kvh) * page_size * D +
                                ((size_t)g * page_size + key % page_size) * 8;
-            Frag8 kf[NKS];
 #pragma unroll
-            for (int ks = 0; ks < NKS; ++ks) kf[ks].u4 = *reinterpret_cast<const uint4 *>(kp + (size_t)ks * 4 * page_size * 8);
-            s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int ks = 0; ks < NKS; ++ks) s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[ks].v, qf[ks].v, s[t], 0, 0, 0);
-        }
-        float sv[8], mx = -INFINITY;
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int key = kstart + 16 * t + 4 * g + i;
-                const bool vis = row_valid && mapped[t] && key <= my_pos && (key >= my_lo || key < keep_first) &&
-                                 key >= k_begin && key < k_end;
-                const float x = vis ? s[t][i] * scale2 : -INFINITY;
-                sv[t * 4 + i] = x;
-                mx = fmaxf(mx, x);
-            }
-        const float m_new = fmaxf(m, quad_rows_max(mx));
-        const float ref = (m_new == -INFINITY) ? 0.f : m_new;
-        const float corr = __builtin_amdgcn_exp2f(m - ref);
-        l *= corr;
-#pragma unroll
-        for (int dt = 0; dt < NDT; ++dt) {
-            o[dt][0] *= corr; o[dt][1] *= corr; o[dt][2] *= corr; o[dt][3] *= corr;
-        }
-        m = m_new;
-        Frag8 pf;
-#pragma unroll
-        for (int j = 0; j < 8; j += 2) {
-            const float p0 = __builtin_amdgcn_exp2f(sv[j] - ref), p1 = __builtin_amdgcn_exp2f(sv[j + 1] - ref);
-            l += p0 + p1;
-            pf.p2[j / 2] = pack_bf16(p0, p1);
-        }
-        uint2 keep[2];
-        const bf16_t *vrow[2];
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
+            for (int ks = 0; ks < NKS; ++ks) kf[t][ks].u4 = *reinterpret_cast<const uint4 *>(kp + (size_t)ks * 4 * page_size * 8);
+            // values: lane (element r of a tile, group g) takes keys 4 g .. 4 g + 3 of the 16-key tile
             const int key0 = kstart + 16 * t + 4 * g;
             int n = min(item_hi + 1, k_end) - key0;
             if (!mapped[t] || key0 + 4 <= k_begin) n = 0;
@@ -414,54 +399,100 @@ gqa_attention_rows_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, 
                 const uint2 head = keep_first_keys(make_uint2(~0u, ~0u), k_begin - key0);
                 keep[t].x &= ~head.x; keep[t].y &= ~head.y;
             }
-            vrow[t] = v_cache + (((size_t)page[t] * kv_heads + kvh) * DV + r) * page_size + key0 % page_size;
+            const bf16_t *vrow = v_cache + (((size_t)page[t] * kv_heads + kvh) * DV + r) * page_size + key0 % page_size;
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt) vv[dt].u2[t] = *reinterpret_cast<const uint2 *>(vrow + (size_t)dt * 16 * page_size);
         }
-        constexpr int VC = NDT < 8 ? NDT : 8;                          // value tiles asked for together
+        __builtin_amdgcn_sched_barrier(0);
+        // a block that every row of the item sees whole needs no mask (wave-uniform)
+        const bool whole = mapped[0] && mapped[1] && kstart >= k_begin && kstart + 32 <= k_end && kstart + 31 <= pos_lo &&
+                           (kstart >= hi_lo || kstart + 32 <= keep_first);
+        Frag8 pf[RT];
 #pragma unroll
-        for (int d0 = 0; d0 < NDT; d0 += VC) {
-            Frag8 vv[VC];
+        for (int rt = 0; rt < RT; ++rt) {
+            f32x4 s[2];
 #pragma unroll
-            for (int j = 0; j < VC; ++j) {
-                vv[j].u2[0] = *reinterpret_cast<const uint2 *>(vrow[0] + (size_t)(d0 + j) * 16 * page_size);
-                vv[j].u2[1] = *reinterpret_cast<const uint2 *>(vrow[1] + (size_t)(d0 + j) * 16 * page_size);
+            for (int t = 0; t < 2; ++t) {
+                s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < NKS; ++ks)
+                    s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t][ks].v, qf[rt][ks].v, s[t], 0, 0, 0);
             }
-            __builtin_amdgcn_sched_barrier(0);
+            float sv[8], mx = -INFINITY;
 #pragma unroll
-            for (int j = 0; j < VC; ++j) {
-                vv[j].u2[0].x &= keep[0].x; vv[j].u2[0].y &= keep[0].y;
-                vv[j].u2[1].x &= keep[1].x; vv[j].u2[1].y &= keep[1].y;
-                o[d0 + j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv[j].v, pf.v, o[d0 + j], 0, 0, 0);
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float x = s[t][i] * scale2;
+                    if (!whole) {
+                        const int key = kstart + 16 * t + 4 * g + i;
+                        const bool vis = row_valid[rt] && mapped[t] && key <= my_pos[rt] &&
+                                         (key >= my_lo[rt] || key < keep_first) && key >= k_begin && key < k_end;
+                        x = vis ? x : -INFINITY;
+                    }
+                    sv[t * 4 + i] = x;
+                    mx = fmaxf(mx, x);
+                }
+            const float bm = quad_rows_max(mx);
+            if (__builtin_amdgcn_ballot_w64(bm > m[rt]) != 0) {       // the maximum moved: re-base l and O
+                const float m_new = fmaxf(m[rt], bm);
+                const float corr = __builtin_amdgcn_exp2f(m[rt] - ((m_new == -INFINITY) ? 0.f : m_new));
+                l[rt] *= corr;
+#pragma unroll
+                for (int dt = 0; dt < NDT; ++dt) {
+                    o[rt][dt][0] *= corr; o[rt][dt][1] *= corr; o[rt][dt][2] *= corr; o[rt][dt][3] *= corr;
+                }
+                m[rt] = m_new;
+            }
+            const float ref = (m[rt] == -INFINITY) ? 0.f : m[rt];
+#pragma unroll
+            for (int j = 0; j < 8; j += 2) {
+                const float p0 = __builtin_amdgcn_exp2f(sv[j] - ref), p1 = __builtin_amdgcn_exp2f(sv[j + 1] - ref);
+                l[rt] += p0 + p1;
+                pf[rt].p2[j / 2] = pack_bf16(p0, p1);
             }
         }
-    }
-    l = quad_rows_sum(l);
-    if (!row_valid) return;
-    const size_t my_global = my_token * heads + my_head;           // row of the output, of the partial results
-    if (splits > 1) {
-        float *po = part_o + (my_global * splits + split) * DV + 4 * g;
 #pragma unroll
-        for (int dt = 0; dt < NDT; ++dt) *reinterpret_cast<float4 *>(po + 16 * dt) = make_float4(o[dt][0], o[dt][1], o[dt][2], o[dt][3]);
-        if (g == 0) {
-            part_ml[(my_global * splits + split) * 2] = m;
-            part_ml[(my_global * splits + split) * 2 + 1] = l;
+        for (int dt = 0; dt < NDT; ++dt) {
+            Frag8 v = vv[dt];
+            v.u2[0].x &= keep[0].x; v.u2[0].y &= keep[0].y;
+            v.u2[1].x &= keep[1].x; v.u2[1].y &= keep[1].y;
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v.v, pf[rt].v, o[rt][dt], 0, 0, 0);
         }
-        return;
     }
-    float mul = 1.f;
-    if (sinks) {
-        const float sk = sinks[my_head] * LAT_LOG2E, m_new = fmaxf(m, sk);
-        const float corr = __builtin_amdgcn_exp2f(m - m_new);
-        l = l * corr + __builtin_amdgcn_exp2f(sk - m_new);
-        mul = corr;
-    }
-    mul /= l;
-    bf16_t *orow = out + my_global * DV + 4 * g;
 #pragma unroll
-    for (int dt = 0; dt < NDT; ++dt) {
-        Frag4 w;
-        w.h[0] = float_to_bf16_bits(o[dt][0] * mul); w.h[1] = float_to_bf16_bits(o[dt][1] * mul);
-        w.h[2] = float_to_bf16_bits(o[dt][2] * mul); w.h[3] = float_to_bf16_bits(o[dt][3] * mul);
-        *reinterpret_cast<uint2 *>(orow + 16 * dt) = w.u2;
+    for (int rt = 0; rt < RT; ++rt) {
+        float lsum = quad_rows_sum(l[rt]);
+        if (!row_valid[rt]) continue;
+        const size_t my_global = my_token[rt] * heads + my_head[rt];   // row of the output, of the partial results
+        if (splits > 1) {
+            float *po = part_o + (my_global * splits + split) * DV + 4 * g;
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt)
+                *reinterpret_cast<float4 *>(po + 16 * dt) = make_float4(o[rt][dt][0], o[rt][dt][1], o[rt][dt][2], o[rt][dt][3]);
+            if (g == 0) {
+                part_ml[(my_global * splits + split) * 2] = m[rt];
+                part_ml[(my_global * splits + split) * 2 + 1] = lsum;
+            }
+            continue;
+        }
+        float mul = 1.f;
+        if (sinks) {
+            const float sk = sinks[my_head[rt]] * LAT_LOG2E, m_new = fmaxf(m[rt], sk);
+            const float corr = __builtin_amdgcn_exp2f(m[rt] - m_new);
+            lsum = lsum * corr + __builtin_amdgcn_exp2f(sk - m_new);
+            mul = corr;
+        }
+        mul /= lsum;
+        bf16_t *orow = out + my_global * DV + 4 * g;
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt) {
+            Frag4 w;
+            w.h[0] = float_to_bf16_bits(o[rt][dt][0] * mul); w.h[1] = float_to_bf16_bits(o[rt][dt][1] * mul);
+            w.h[2] = float_to_bf16_bits(o[rt][dt][2] * mul); w.h[3] = float_to_bf16_bits(o[rt][dt][3] * mul);
+            *reinterpret_cast<uint2 *>(orow + 16 * dt) = w.u2;
+        }
     }
 }
 
@@ -482,7 +513,8 @@ extern "C" int kva_attention_rows_mfma(void *out, float *part_o, float *part_ml,
                                        const int *entry_seat, const int *entry_q_start, const int *entry_start_pos,
                                        int num_items, int total_rows, int heads, int kv_heads, int head_dim,
                                        int value_dim, int page_size, float scale, int window, int keep_first,
-                                       const float *sinks, int splits, int per_split, hipStream_t stream) {
+                                       const float *sinks, int splits, int per_split, int row_tiles,
+                                       hipStream_t stream) {
     KVA_REQUIRE(kva_attention_rows_mfma_supported(head_dim, value_dim, page_size),
                 "attention_rows_mfma: no instance for keys of %d, values of %d, pages of %d", head_dim, value_dim, page_size);
     KVA_REQUIRE(num_items >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && max_blocks > 0 && total_rows >= 0,
@@ -492,13 +524,19 @@ extern "C" int kva_attention_rows_mfma(void *out, float *part_o, float *part_ml,
                     (splits == 1 || (per_split > 0 && per_split % 32 == 0 && part_o && part_ml)),
                 "attention_rows_mfma: key ranges need a length that is a multiple of 32 and a workspace");
     KVA_REQUIRE(window >= 0 && keep_first >= 0, "attention_rows_mfma: negative window or kept first positions");
+    KVA_REQUIRE(row_tiles == 1 || (row_tiles == 2 && value_dim <= 128 && head_dim <= 128),
+                "attention_rows_mfma: one row tile an item, or two for heads up to 128");
     if (window == 0) keep_first = 0;
     if (num_items == 0) return KVA_OK;
     dim3 grid(num_items, kv_heads * splits), block(KVA_WAVE);
     bool done = false;
 #define LAUNCH_ONE(NDT, NKS)                                                                                    \
     if (!done && value_dim == NDT * 16 && head_dim == NKS * 32) {                                               \
-        hipLaunchKernelGGL((gqa_attention_rows_kernel<NDT, NKS>), grid, block, 0, stream, (bf16_t *)out, part_o, \
+        auto kernel = gqa_attention_rows_kernel<NDT, NKS, 1>;                                                    \
+        if constexpr (NDT <= 8 && NKS <= 4) {                                                                    \
+            if (row_tiles == 2) kernel = gqa_attention_rows_kernel<NDT, NKS, 2>;                                 \
+        }                                                                                                        \
+        hipLaunchKernelGGL(kernel, grid, block, 0, stream, (bf16_t *)out, part_o,                                \
                            part_ml, (const bf16_t *)q, q_stride, (const bf16_t *)k_cache,                        \
                            (const bf16_t *)v_cache, block_table, max_blocks, item_entry, item_row0, entry_seat,  \
                            entry_q_start, entry_start_pos, heads, kv_heads, page_size, scale, window,            \

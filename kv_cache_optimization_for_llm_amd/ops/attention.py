@@ -69,6 +69,9 @@ _LDS_TARGET_GROUPS = 1024
 _LDS_MIN_KEYS_PER_SPLIT = 1024
 
 
+_ROWS_TWO_TILES = 32 * 1024          # (token, head) rows of a step from which the general rows kernel takes two tiles an item
+
+
 def use_lds_kernel(groups: int, mean_keys: float, head_dim: int) -> bool:
     """Whether prompt rows that make ``groups`` workgroups of 128 rows (over all kv heads) and visit
     ``mean_keys`` keys each on average go to the workgroup kernel."""
@@ -380,14 +383,18 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
         if qkv.dtype == torch.bfloat16 and qkv.shape[1] % 8 == 0 \
                 and K.attention_rows_mfma_supported(head_dim, value_dim, kv.page_size):
             from .latent_attention import choose_ranges
-            item_entry, item_row0, _ = batch.attention_items(num_q_heads // num_kv_heads, 1, "all")
+            # prompt portions with enough rows to fill the chip: two row tiles an item share their loads
+            group = num_q_heads // num_kv_heads
+            tiles = 2 if (head_dim <= 128 and value_dim <= 128
+                          and batch.num_tokens * group * num_kv_heads >= _ROWS_TWO_TILES) else 1
+            item_entry, item_row0, _ = batch.attention_items(group, tiles, "all")
             # (with a window most ranges of a long context hold no visible key: their wavefronts end at once)
             ranges, per = choose_ranges(item_entry.shape[0] * num_kv_heads, batch.max_context,
                                         window + keep_first if window > 0 else 0)
             return K.attention_rows_mfma(qkv, qkv.shape[1], out, kv.k_cache, kv.v_cache, kv.block_table, item_entry,
                                          item_row0, batch.entry_seat, batch.entry_q_start, batch.entry_start_pos,
                                          num_q_heads, num_kv_heads, head_dim, scale, window, keep_first, sinks,
-                                         value_dim, ranges, per)
+                                         value_dim, ranges, per, tiles)
         return K.attention_rowwise(qkv, qkv.shape[1], out, kv.k_cache, kv.v_cache, kv.block_table,
                                    batch.tok_seat, batch.positions, num_q_heads, num_kv_heads,
                                    head_dim, scale, window, keep_first, sinks, value_dim)

@@ -476,10 +476,12 @@ def attention_rows_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k
                         item_row0: torch.Tensor, entry_seat: torch.Tensor, entry_q_start: torch.Tensor,
                         entry_start_pos: torch.Tensor, num_q_heads: int, num_kv_heads: int, head_dim: int,
                         scale: float, window: int = 0, keep_first: int = 0, sinks: Optional[torch.Tensor] = None,
-                        value_dim: Optional[int] = None, splits: int = 1, per_split: int = 0) -> torch.Tensor:
-    """:func:`attention_rowwise` with all its options on the matrix cores (bf16): a work item is 16
-    rows ``token_in_entry * group + head_in_group`` of entry ``item_entry[i]`` from ``item_row0[i]``
-    on, for every kv head; with ``splits`` > 1 the keys are cut into ranges of ``per_split`` and a
+                        value_dim: Optional[int] = None, splits: int = 1, per_split: int = 0,
+                        row_tiles: int = 1) -> torch.Tensor:
+    """:func:`attention_rowwise` with all its options on the matrix cores (bf16): a work item is
+    ``16 * row_tiles`` rows ``token_in_entry * group + head_in_group`` of entry ``item_entry[i]`` from
+    ``item_row0[i]`` on, for every kv head (two row tiles, for heads up to 128, share what a
+    wavefront loads); with ``splits`` > 1 the keys are cut into ranges of ``per_split`` and a
     second kernel adds the ranges' results up."""
     tokens = out.shape[0]
     value_dim = head_dim if value_dim is None else int(value_dim)
@@ -510,7 +512,7 @@ def attention_rows_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k
         _dev(entry_seat, "entry_seat", torch.int32), _dev(entry_q_start, "entry_q_start", torch.int32),
         _dev(entry_start_pos, "entry_start_pos", torch.int32), n, tokens * num_q_heads, num_q_heads, num_kv_heads,
         head_dim, value_dim, page_size, float(scale), int(window), int(keep_first), _opt(sinks, "sinks"), int(splits),
-        int(per_split), _stream()), "attention_rows_mfma")
+        int(per_split), int(row_tiles), _stream()), "attention_rows_mfma")
     return out
 
 

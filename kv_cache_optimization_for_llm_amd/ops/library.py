@@ -53,7 +53,7 @@ _HIP_SIGNATURES = {
     "kva_latent_encode_cache": [P, I, I, P, P, P, I, P, I, F, P, P, P, P, I, I, I, I, I, I, I, P],
     "kva_latent_attention_mfma_supported": [I, I, I],
     "kva_attention_rows_mfma_supported": [I, I, I],
-    "kva_attention_rows_mfma": [P, P, P, P, I, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P, I, I, P],
+    "kva_attention_rows_mfma": [P, P, P, P, I, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P, I, I, I, P],
     "kva_latent_attention_mfma": [P, P, P, P, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P, I, I, P],
     "kva_heads_matmul": [P, I, I, P, I, I, P, I, I, I, I, P, I, I, P],
     "kva_heads_matmul_mfma_supported": [I, I, I],

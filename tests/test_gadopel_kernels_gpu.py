@@ -304,10 +304,11 @@ def test_latent_attention_on_the_matrix_cores(heads, rank, rot, window, keep_fir
         close(out, want_all[start:upto], 3e-2, f"entry {start}+{n}")
 
 
+@pytest.mark.parametrize("row_tiles", [1, 2])
 @pytest.mark.parametrize("per_range", [0, 64])
 @pytest.mark.parametrize("heads, kv_heads, dim, vdim, window, keep_first", [
     (4, 1, 64, 64, 40, 20), (8, 2, 32, 64, 33, 17), (6, 3, 64, 32, 0, 0), (32, 2, 64, 64, 16, 16), (2, 2, 128, 128, 50, 0)])
-def test_windowed_attention_on_the_matrix_cores(heads, kv_heads, dim, vdim, window, keep_first, per_range, gpu):
+def test_windowed_attention_on_the_matrix_cores(heads, kv_heads, dim, vdim, window, keep_first, per_range, row_tiles, gpu):
     """The matrix-core kernel that takes a window with kept first positions, sinks and a value
     size of its own: portions of prompts and decoded tokens against the plain attention."""
     page, scale, length = 16, 0.2, 200
@@ -330,11 +331,12 @@ def test_windowed_attention_on_the_matrix_cores(heads, kv_heads, dim, vdim, wind
         v_cache[sl // page, :, :, sl % page] = v_all[:upto].to(gpu)
         k_cache = K.keys_to_pages(kp)
         q = q_all[start:upto].reshape(n, heads * dim).contiguous().to(gpu)
-        tiles = (n * group + 15) // 16
+        per_item = 16 * row_tiles
+        tiles = (n * group + per_item - 1) // per_item
         out = torch.empty((n, heads * vdim), dtype=torch.bfloat16, device=gpu)
         ranges = 1 if per_range == 0 else -(-upto // per_range)
         K.attention_rows_mfma(q, heads * dim, out, k_cache, v_cache, table.to(gpu), i32([0] * tiles),
-                              i32([16 * t for t in range(tiles)]), i32([1]), i32([0, n]), i32([start]), heads, kv_heads,
-                              dim, scale, window, keep_first, sinks.to(gpu), vdim, ranges, per_range)
+                              i32([per_item * t for t in range(tiles)]), i32([1]), i32([0, n]), i32([start]), heads, kv_heads,
+                              dim, scale, window, keep_first, sinks.to(gpu), vdim, ranges, per_range, row_tiles)
         assert torch.isfinite(out.float()).all(), f"entry {start}+{n}"
         close(out.view(n, heads, vdim), want_all[start:upto], 3e-2, f"entry {start}+{n}")
