@@ -81,6 +81,9 @@ class GadopelConfig:
                     raise ConfigError(f"config.json: {where}: {m['heads']} heads is not a multiple of {g} kv heads")
                 if rot["dims"] > m["dim"]:
                     raise ConfigError(f"config.json: {where}: rot.dims {rot['dims']} exceeds dim {m['dim']}")
+                if m["dim"] % 4:
+                    raise ConfigError(f"config.json: {where}: dim {m['dim']} must be a multiple of 4 (keys lie in the "
+                                      "cache in chunks of 4 or 8 elements)")
                 if m.get("mask") is not None:
                     _need(m["mask"], "size", where + ".mixer.mask")
             mlp = layer.get("mlp")

@@ -31,7 +31,7 @@ def engine_for(folder, dtype, **kw):
     return Engine(folder, EngineOptions(**opts))
 
 
-REQUESTS = {"P": [1, 2, 9, 40, 77], "Q": [3, 33, 70], "R": [1, 18, 50, 131]}
+REQUESTS = {"P": [1, 2, 9, 40, 77], "Q": [3, 33, 70], "R": [1, 18, 50, 131], "S": [1, 5, 47, 150]}
 
 
 def requests_for(name, cfg):
@@ -39,7 +39,7 @@ def requests_for(name, cfg):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["P", "Q", "R"])
+@pytest.mark.parametrize("name", ["P", "Q", "R", "S"])
 def test_whole_prompts_and_the_first_tokens(name, dtype, models, gpu):
     cfg, folder, state = models[name]
     reqs = requests_for(name, cfg)
@@ -52,7 +52,7 @@ def test_whole_prompts_and_the_first_tokens(name, dtype, models, gpu):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["P", "Q", "R"])
+@pytest.mark.parametrize("name", ["P", "Q", "R", "S"])
 def test_prefill_against_token_by_token_decoding(name, dtype, models, gpu):
     """Most of a request in one step, the rest one token at a time: long enough that every window
     passes over decoded tokens and leaves the kept first positions behind."""
@@ -70,7 +70,7 @@ def test_prefill_against_token_by_token_decoding(name, dtype, models, gpu):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("sizes", [(2,), (7, 16, 5, 2, 33, 3, 64, 2), (17, 1, 1, 30)])
-@pytest.mark.parametrize("name", ["P", "R"])
+@pytest.mark.parametrize("name", ["P", "R", "S"])
 def test_portions_of_any_size(name, sizes, dtype, models, gpu):
     cfg, folder, state = models[name]
     reqs = {k: v for k, v in requests_for(name, cfg).items() if len(v) > 8}
@@ -81,7 +81,7 @@ def test_portions_of_any_size(name, sizes, dtype, models, gpu):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name, seed", [("P", 0), ("Q", 1), ("R", 2), ("R", 3)])
+@pytest.mark.parametrize("name, seed", [("P", 0), ("Q", 1), ("R", 2), ("R", 3), ("S", 4), ("S", 5)])
 def test_mixed_batches_on_a_small_pool_reuse_pages_and_seats(name, seed, dtype, models, gpu):
     cfg, folder, state = models[name]
     lengths = [40, 3, 90, 25, 61, 2, 130, 47, 33]
@@ -144,7 +144,7 @@ def test_the_trace_runner_replays_a_mixed_schedule(dtype, models, tmp_path, gpu)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["P", "R"])
+@pytest.mark.parametrize("name", ["P", "R", "S"])
 def test_greedy_generation_through_the_entry_point(name, dtype, models, gpu):
     cfg, folder, state = models[name]
     prompts = [U.prompt(cfg, n, 3 + n) for n in (1, 12, 37, 64, 5, 90)]
@@ -163,9 +163,10 @@ def test_greedy_generation_through_the_entry_point(name, dtype, models, gpu):
     assert llm.engine.cache.free_seats == 3
 
 
-def test_decode_steps_from_graphs_equal_eager_steps(models, gpu):
+@pytest.mark.parametrize("name", ["R", "S"])
+def test_decode_steps_from_graphs_equal_eager_steps(name, models, gpu):
     """A bf16 decode step replayed from its HIP graph gives bit for bit what the eager step gives."""
-    cfg, folder, state = models["R"]
+    cfg, folder, state = models[name]
     reqs = {f"g{i}": U.prompt(cfg, n, 31 + i) for i, n in enumerate([48, 80])}
     steps = R.tail_decoded(reqs, tail=20)
     eager = U.run_steps(engine_for(folder, "bfloat16", use_graphs=False), steps)
@@ -175,3 +176,36 @@ def test_decode_steps_from_graphs_equal_eager_steps(models, gpu):
     assert eng.graphs.replays > 0
     for key in eager:
         np.testing.assert_array_equal(eager[key], replayed[key], err_msg=str(key))
+
+
+def test_portion_steps_from_graphs_equal_eager_steps(models, gpu, monkeypatch):
+    """Steps with prompt portions whose shape comes back run from a graph of their own: the same
+    portions of two requests beside each other, four times over, eagerly and replayed.  (A graph
+    cuts the keys into ranges by its context bucket, an eager step by the context it sees: the
+    eager steps are given the bucket too, and then a replay is bit for bit the eager step.)"""
+    import kv_cache_optimization_for_llm_amd.engine.engine as engine_module
+    from kv_cache_optimization_for_llm_amd.engine.graphs import context_bucket
+    plain_build = engine_module.build_batch
+
+    def build_with_bucket(*args, **kwargs):
+        batch = plain_build(*args, **kwargs)
+        batch.max_context = context_bucket(batch.max_context)
+        return batch
+    monkeypatch.setattr(engine_module, "build_batch", build_with_bucket)
+    cfg, folder, state = models["S"]
+    steps, n = [], 0
+    for rep in range(4):
+        reqs = {f"a{rep}": U.prompt(cfg, 96, 60 + rep), f"b{rep}": U.prompt(cfg, 96, 70 + rep)}
+        for lo in range(0, 96, 24):
+            steps.append({"step": n, "entries": [{"id": rid, "tokens": toks[lo:lo + 24], "want": [0, 23]}
+                                                  for rid, toks in reqs.items()],
+                          "end": list(reqs) if lo == 72 else []})
+            n += 1
+    eager = U.run_steps(engine_for(folder, "bfloat16", use_graphs=False), steps)
+    eng = engine_for(folder, "bfloat16")
+    replayed = U.run_steps(eng, steps)
+    assert eng.portion_graphs is not None and eng.portion_graphs.replays > 0
+    for key in eager:
+        np.testing.assert_array_equal(eager[key], replayed[key], err_msg=str(key))
+    reqs = {f"{c}{rep}": U.prompt(cfg, 96, (60 if c == "a" else 70) + rep) for rep in range(4) for c in "ab"}
+    U.assert_rows(replayed, U.expected_rows(cfg, state, reqs), "bfloat16", "replayed portions")
