@@ -57,8 +57,10 @@ def main(argv=None) -> int:
         prompts = prompts[:args.num_prompts]
     else:
         import numpy as np
-        with open(os.path.join(args.model_dir, "config.json")) as f:
-            vocab = json.load(f)["vocab_size"]
+        # the vocabulary's size as the folder's architecture reads it from its own configuration keys
+        from ..config.model_config import read_config_json
+        from ..models.builder import spec_for_config
+        vocab = spec_for_config(read_config_json(args.model_dir))[1].vocab_size
         rng = np.random.default_rng(args.seed)
         prompts = [[int(t) for t in rng.integers(0, vocab, args.prompt_len)] for _ in range(args.num_prompts)]
 

@@ -67,13 +67,16 @@ def run_one(args, shape: str, batch: int, mode: str) -> dict:
     from ..ops.gemm_bf16 import decode_tune_rows
 
     cfg = dict(SHAPES[shape]) if shape in SHAPES else json.load(open(shape))
-    full_layers = cfg["num_hidden_layers"]
-    if args.layers:
+    # (a configuration file of another architecture names its layers one by one: it runs whole,
+    # and what a step reads is taken from the engine's own tensors and cache entry)
+    llama_keys = "num_hidden_layers" in cfg
+    full_layers = cfg["num_hidden_layers"] if llama_keys else len(cfg.get("layers", ()))
+    if args.layers and llama_keys:
         cfg["num_hidden_layers"] = min(args.layers, full_layers)
     longest = args.prompt_len + args.new_tokens + 1
     if shape in SHAPES:
         cfg["max_position_embeddings"] = max(2048, 1 << (longest - 1).bit_length())
-    elif longest > cfg["max_position_embeddings"]:
+    elif "max_position_embeddings" in cfg and longest > cfg["max_position_embeddings"]:
         raise SystemExit(f"{shape}: prompts of {args.prompt_len} plus {args.new_tokens} new tokens do not fit "
                          f"max_position_embeddings {cfg['max_position_embeddings']}")
     seats = min(batch, args.max_seqs) if args.max_seqs else batch
@@ -105,7 +108,12 @@ def run_one(args, shape: str, batch: int, mode: str) -> dict:
     decode_steps = decode_tokens = seen_decode_steps = 0
     decode_time = 0.0
     decode_bytes = 0.0
-    wbytes, kvbytes = weight_bytes(cfg), kv_bytes_per_token(cfg)
+    if llama_keys:
+        wbytes, kvbytes = weight_bytes(cfg), kv_bytes_per_token(cfg)
+    else:
+        mats = [lin.weight for lin in engine.model.linears()] + [engine.model.head.weight]
+        wbytes = sum(t.numel() * t.element_size() for t in mats)
+        kvbytes = engine.cache.page_bytes() // args.page_size
     reasons: Dict[str, int] = {}
     torch.cuda.synchronize()
     t_start = time.perf_counter()
@@ -144,7 +152,7 @@ def run_one(args, shape: str, batch: int, mode: str) -> dict:
     st = engine.cache.stats()
     engine.cache.check()
     out = {
-        "shape": shape, "layers": cfg["num_hidden_layers"], "layers_full": full_layers, "batch": batch,
+        "shape": shape, "layers": cfg["num_hidden_layers"] if llama_keys else full_layers, "layers_full": full_layers, "batch": batch,
         "cache_mode": mode, "reserve_policy": args.reserve_policy if mode == "contiguous" else None,
         "workload": args.workload, "prompt_tokens": sum(lens), "new_tokens_each": args.new_tokens,
         "seats": seats, "cache_tokens": st["kv_tokens_total"],
