@@ -97,48 +97,54 @@ extern "C" int kva_heads_matmul(void *out, int o_row, int o_head, const void *x,
 // bytes of its row.  K = 32 NKS.  blockIdx: (n tile, head, group of row tiles).
 #include "attention_frag.h"
 
-template <int NKS>
+template <int NKS, int NT>
 __global__ void __launch_bounds__(KVA_WAVE)
 heads_matmul_mfma_kernel(bf16_t *__restrict__ out, int o_row, int o_head, const bf16_t *__restrict__ x, int x_row,
                          int x_head, const bf16_t *__restrict__ w, int M, int N, int tiles_per_wave,
                          const bf16_t *__restrict__ gate, int g_row) {
+    // NT neighbouring tiles of 16 outputs a wavefront: every fragment of x it loads serves NT products
+    // (many rows: what a wavefront takes in per product is what bounds it); NT = 1 for few rows,
+    // where more wavefronts matter more
     constexpr int K = NKS * 32;
     const int lane = threadIdx.x, r = lane & 15, g = lane >> 4;
-    const int n0 = blockIdx.x * 16, h = blockIdx.y;
-    Frag8 wf[NKS];
-    {
-        const int n = min(n0 + r, N - 1);
+    const int n_first = blockIdx.x * 16 * NT, h = blockIdx.y;
+    Frag8 wf[NT][NKS];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const int n = min(n_first + 16 * nt + r, N - 1);
         const bf16_t *wrow = w + ((size_t)h * N + n) * K + 8 * g;
 #pragma unroll
-        for (int ks = 0; ks < NKS; ++ks) wf[ks].u4 = *reinterpret_cast<const uint4 *>(wrow + 32 * ks);
+        for (int ks = 0; ks < NKS; ++ks) wf[nt][ks].u4 = *reinterpret_cast<const uint4 *>(wrow + 32 * ks);
     }
     const int first = blockIdx.z * tiles_per_wave;
     for (int tile = first; tile < first + tiles_per_wave && tile * 16 < M; ++tile) {
         const int t = min(tile * 16 + r, M - 1);
         const bf16_t *xrow = x + (size_t)t * x_row + (size_t)h * x_head + 8 * g;
-        f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+        Frag8 xf[NKS];
 #pragma unroll
-        for (int ks = 0; ks < NKS; ++ks) {
-            Frag8 xf;
-            xf.u4 = *reinterpret_cast<const uint4 *>(xrow + 32 * ks);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[ks].v, xf.v, acc, 0, 0, 0);
-        }
-        // lane (row t = r, group g) holds outputs n0 + 4 g .. + 3 of its row
-        if (gate) {
-            const float gmul = 1.0f / (1.0f + expf(-to_float(gate[(size_t)t * g_row + h])));
-            acc[0] *= gmul; acc[1] *= gmul; acc[2] *= gmul; acc[3] *= gmul;
-        }
-        if (tile * 16 + r < M) {
-            bf16_t *o = out + (size_t)t * o_row + (size_t)h * o_head + n0 + 4 * g;
-            if (n0 + 4 * g + 3 < N && ((o_row | o_head) % 4 == 0)) {
-                Frag4 v;
+        for (int ks = 0; ks < NKS; ++ks) xf[ks].u4 = *reinterpret_cast<const uint4 *>(xrow + 32 * ks);
+        float gmul = 1.f;
+        if (gate) gmul = 1.0f / (1.0f + expf(-to_float(gate[(size_t)t * g_row + h])));
 #pragma unroll
-                for (int i = 0; i < 4; ++i) v.h[i] = float_to_bf16_bits(acc[i]);
-                *reinterpret_cast<uint2 *>(o) = v.u2;
-            } else {
+        for (int nt = 0; nt < NT; ++nt) {
+            const int n0 = n_first + 16 * nt;
+            if (n0 >= N) break;
+            f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    if (n0 + 4 * g + i < N) o[i].bits = float_to_bf16_bits(acc[i]);
+            for (int ks = 0; ks < NKS; ++ks) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[nt][ks].v, xf[ks].v, acc, 0, 0, 0);
+            // lane (row t = r, group g) holds outputs n0 + 4 g .. + 3 of its row
+            if (tile * 16 + r < M) {
+                bf16_t *o = out + (size_t)t * o_row + (size_t)h * o_head + n0 + 4 * g;
+                if (n0 + 4 * g + 3 < N && ((o_row | o_head) % 4 == 0)) {
+                    Frag4 v;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) v.h[i] = float_to_bf16_bits(acc[i] * gmul);
+                    *reinterpret_cast<uint2 *>(o) = v.u2;
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        if (n0 + 4 * g + i < N) o[i].bits = float_to_bf16_bits(acc[i] * gmul);
+                }
             }
         }
     }
@@ -164,15 +170,22 @@ extern "C" int kva_heads_matmul_mfma(void *out, int o_row, int o_head, const voi
                 "heads_matmul_mfma: strides do not fit %d heads of %d -> %d", heads, K, N);
     if (rows == 0) return KVA_OK;
     const int row_tiles = (rows + 15) / 16;
-    // enough wavefronts to fill the chip before a wavefront takes more than one row tile
-    int per_wave = 1;
-    while (per_wave < 8 && (long long)((N + 15) / 16) * heads * ((row_tiles + per_wave - 1) / per_wave) > 4096) per_wave *= 2;
-    dim3 grid((N + 15) / 16, heads, (row_tiles + per_wave - 1) / per_wave), block(KVA_WAVE);
-    KVA_REQUIRE(grid.z <= 65535, "heads_matmul_mfma: %d rows are too many for one launch", rows);
+    const int n_tiles = (N + 15) / 16;
+    // many rows: several output tiles a wavefront (at most 32 fragments of W in its registers)
+    const bool wide = rows > 64;
     bool done = false;
 #define LAUNCH_ONE(NKS)                                                                                          \
     if (!done && K == NKS * 32) {                                                                                \
-        hipLaunchKernelGGL(heads_matmul_mfma_kernel<NKS>, grid, block, 0, stream, (bf16_t *)out, o_row, o_head,  \
+        constexpr int NTW = NKS <= 8 ? 4 : (NKS <= 16 ? 2 : 1);                                                  \
+        const int nt = wide ? NTW : 1;                                                                           \
+        const int groups = (n_tiles + nt - 1) / nt;                                                              \
+        /* enough wavefronts to fill the chip before a wavefront takes more than one row tile */                 \
+        int per_wave = 1;                                                                                        \
+        while (per_wave < 8 && (long long)groups * heads * ((row_tiles + per_wave - 1) / per_wave) > 4096) per_wave *= 2; \
+        dim3 grid(groups, heads, (row_tiles + per_wave - 1) / per_wave), block(KVA_WAVE);                        \
+        KVA_REQUIRE(grid.z <= 65535, "heads_matmul_mfma: %d rows are too many for one launch", rows);            \
+        auto kernel = wide ? heads_matmul_mfma_kernel<NKS, NTW> : heads_matmul_mfma_kernel<NKS, 1>;              \
+        hipLaunchKernelGGL(kernel, grid, block, 0, stream, (bf16_t *)out, o_row, o_head,                         \
                            (const bf16_t *)x, x_row, x_head, (const bf16_t *)w, rows, N, per_wave,               \
                            (const bf16_t *)gate, g_row);                                                         \
         done = true;                                                                                             \
