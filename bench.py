@@ -82,7 +82,7 @@ def gadopel_config(layers: int, vocab: int) -> dict:
                 "mixer": {"heads": 32, "kv_heads": 8, "dim": 64, "vdim": 64, "scale": 1.0,
                           "mask": {"size": 1024, "keep_first": 64},
                           "rot": {"base": 500000.0, "dims": 64,
-                                  "scaling": {"factor": 8.0, "original": 2048, "fast": 32.0, "slow": 1.0}}}}
+                                  "scaling": {"factor": 16.0, "original": 4096, "fast": 16.0, "slow": 2.0}}}}
     return {"architecture": "Gadopel", "vocab": vocab, "width": 2048, "norm": {"eps": 1e-6},
             "layers": [latent if i % 2 == 0 else windowed for i in range(layers)], "max_positions": 8192}
 

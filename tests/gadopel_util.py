@@ -55,7 +55,7 @@ CFG_R = {"architecture": "Gadopel", "vocab": 300, "width": 128, "norm": {"eps": 
 #    under 5 and 20 heads, windowed attention with keys of 64 and values of 64 / 32, a group of 8
 #    query heads a kv head; the loop over the last two layers.
 CFG_S = {"architecture": "Gadopel", "vocab": 257, "width": 256, "norm": {"eps": 1e-6}, "layers": [
-    attention_layer(8, 1, 64, 64, 32, base=100000.0, scale=0.125, mask={"size": 40, "keep_first": 20}, scaling=YARN, ff=320),
+    attention_layer(8, 1, 64, 64, 32, base=100000.0, scale=0.125, mask={"size": 44, "keep_first": 18}, scaling=YARN, ff=320),
     latent_layer(5, 32, 32, 16, 64, scale=0.1, ff=192),
     attention_layer(4, 2, 64, 32, 64, scale=0.125, mask={"size": 21, "keep_first": 2}, ff=256),
     latent_layer(20, 16, 64, 32, 128, base=3000.0, scale=0.09),

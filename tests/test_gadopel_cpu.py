@@ -75,7 +75,7 @@ def test_random_weights_mode_writes_a_folder_the_plain_model_reads(tmp_path):
 
 
 def test_yarn_frequencies_and_magnitude():
-    for dims, base, sc in [(64, 250000.0, dict(factor=8.0, original=2048, fast=32.0, slow=1.0)),
+    for dims, base, sc in [(64, 300000.0, dict(factor=6.0, original=1024, fast=24.0, slow=2.0)),
                            (16, 10000.0, dict(factor=4.0, original=64, fast=8.0, slow=2.0)),
                            (8, 10000.0, dict(factor=16.0, original=32, fast=4.0, slow=1.0))]:
         got = yarn_frequencies(dims, base, **sc)

@@ -135,9 +135,9 @@ def standout(q, k, query_pos, key_pos, head, kv_head, strength=12.0):
 
 CASES = [  # (length, window, keep_first, query position, key that stands out)
     (300, 0, 0, 299, 0), (300, 0, 0, 299, 157),                     # far keys, no window
-    (300, 40, 20, 299, 260), (300, 40, 20, 299, 259),              # just inside / outside the window
-    (300, 40, 20, 299, 19), (300, 40, 20, 299, 20),                # the last kept position / the first that is not
-    (300, 40, 20, 45, 20), (300, 40, 20, 59, 20), (300, 40, 20, 60, 20),
+    (300, 44, 18, 299, 256), (300, 44, 18, 299, 255),              # just inside / outside the window
+    (300, 44, 18, 299, 17), (300, 44, 18, 299, 18),                # the last kept position / the first that is not
+    (300, 44, 18, 45, 18), (300, 44, 18, 61, 18), (300, 44, 18, 62, 18),
     (130, 16, 16, 129, 15), (130, 16, 16, 129, 16), (130, 16, 16, 129, 113), (130, 16, 16, 129, 114),   # page edges
     (70, 64, 0, 69, 5), (70, 64, 0, 69, 6), (5, 3, 1, 4, 0), (5, 3, 1, 4, 1), (1, 0, 0, 0, 0),
 ]
@@ -264,7 +264,7 @@ def test_per_head_products_into_column_ranges(rows, heads, n, k, x_pad, out_pad,
 
 @pytest.mark.parametrize("per_range", [0, 32, 96])
 @pytest.mark.parametrize("heads, rank, rot, window, keep_first", [
-    (3, 64, 32, 0, 0), (16, 64, 64, 0, 0), (5, 128, 32, 40, 20), (20, 64, 32, 33, 0), (6, 128, 64, 16, 16)])
+    (3, 64, 32, 0, 0), (16, 64, 64, 0, 0), (5, 128, 32, 36, 10), (20, 64, 32, 33, 0), (6, 128, 64, 16, 16)])
 def test_latent_attention_on_the_matrix_cores(heads, rank, rot, window, keep_first, per_range, gpu):
     """Entries of a step - two portions of prompts cut in the middle of pages and of tiles, and
     decoded tokens, one right behind a page's edge - against the plain attention over all rows;
@@ -307,7 +307,7 @@ def test_latent_attention_on_the_matrix_cores(heads, rank, rot, window, keep_fir
 @pytest.mark.parametrize("row_tiles", [1, 2])
 @pytest.mark.parametrize("per_range", [0, 64])
 @pytest.mark.parametrize("heads, kv_heads, dim, vdim, window, keep_first", [
-    (4, 1, 64, 64, 40, 20), (8, 2, 32, 64, 33, 17), (6, 3, 64, 32, 0, 0), (32, 2, 64, 64, 16, 16), (2, 2, 128, 128, 50, 0)])
+    (4, 1, 64, 64, 44, 18), (8, 2, 32, 64, 33, 17), (6, 3, 64, 32, 0, 0), (32, 2, 64, 64, 16, 16), (2, 2, 128, 128, 50, 0)])
 def test_windowed_attention_on_the_matrix_cores(heads, kv_heads, dim, vdim, window, keep_first, per_range, row_tiles, gpu):
     """The matrix-core kernel that takes a window with kept first positions, sinks and a value
     size of its own: portions of prompts and decoded tokens against the plain attention."""

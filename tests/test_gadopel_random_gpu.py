@@ -21,7 +21,7 @@ def random_config(seed: int) -> dict:
         if rng.random() < 0.4:
             rank, rot = pick((24, 4), (40, 8), (64, 32), (64, 64), (128, 32), (96, 16), (128, 64), (200, 24))
             layers.append(U.latent_layer(pick(1, 2, 3, 5, 8, 18), pick(8, 16, 24, 32, 64), rot, pick(8, 16, 24, 32, 48),
-                                         rank, base=float(pick(100.0, 10000.0, 250000.0)), scale=pick(0.08, 0.125, 0.2), ff=ff))
+                                         rank, base=float(pick(100.0, 10000.0, 300000.0)), scale=pick(0.08, 0.125, 0.2), ff=ff))
         else:
             kv = pick(1, 2, 3, 4)
             dim = pick(16, 20, 32, 48, 64, 128)
