@@ -23,7 +23,8 @@ qk_encode_cache_kernel(T *__restrict__ qkv, int row_stride, int k_off, int v_off
                        T *__restrict__ v_cache, const float *__restrict__ cos_table,
                        const float *__restrict__ sin_table, const int *__restrict__ positions,
                        const int *__restrict__ slot_mapping, int num_q_heads, int num_kv_heads, int head_dim,
-                       int value_dim, int rot, int interleaved, float unit_eps, int page_size) {
+                       int value_dim, int rot, int interleaved, float unit_eps, int page_size,
+                       const T *__restrict__ bias) {
     const int t = blockIdx.x;
     const int lane = threadIdx.x % KVA_WAVE, wave = threadIdx.x / KVA_WAVE, waves = blockDim.x / KVA_WAVE;
     T *row = qkv + (size_t)t * row_stride;
@@ -38,6 +39,8 @@ qk_encode_cache_kernel(T *__restrict__ qkv, int row_stride, int k_off, int v_off
         const bool is_q = head < num_q_heads;
         if (!is_q && slot < 0) continue;
         T *h = is_q ? row + (size_t)head * head_dim : row + k_off + (size_t)(head - num_q_heads) * head_dim;
+        // (optional) the projection's bias, laid out [q heads | k heads | v heads] without gaps
+        const T *hb = bias ? bias + (size_t)head * head_dim : nullptr;
         float o1[PER], o2[PER];
         int i1[PER], i2[PER];
         float sq = 0.f;
@@ -58,7 +61,8 @@ qk_encode_cache_kernel(T *__restrict__ qkv, int row_stride, int k_off, int v_off
                 i1[c] = rot + 2 * (p - half);
                 i2[c] = i1[c] + 1;
             }
-            const float u = to_float(h[i1[c]]), v = to_float(h[i2[c]]);
+            const float u = to_float(h[i1[c]]) + (hb ? to_float(hb[i1[c]]) : 0.f);
+            const float v = to_float(h[i2[c]]) + (hb ? to_float(hb[i2[c]]) : 0.f);
             if (p < half) {
                 const float co = cs[p], si = sn[p];
                 o1[c] = u * co - v * si;
@@ -90,9 +94,11 @@ qk_encode_cache_kernel(T *__restrict__ qkv, int row_stride, int k_off, int v_off
     }
     if (slot >= 0) {
         const T *v = row + v_off;
+        const T *vb = bias ? bias + (size_t)(num_q_heads + num_kv_heads) * head_dim : nullptr;
         for (int w = threadIdx.x; w < num_kv_heads * value_dim; w += blockDim.x) {
             const int kvh = w / value_dim, j = w % value_dim;
-            v_cache[(((size_t)page * num_kv_heads + kvh) * value_dim + j) * page_size + off] = v[w];
+            v_cache[(((size_t)page * num_kv_heads + kvh) * value_dim + j) * page_size + off] =
+                vb ? from_float<T>(to_float(v[w]) + to_float(vb[w])) : v[w];
         }
     }
 }
@@ -170,7 +176,7 @@ extern "C" int kva_qk_encode_cache(void *qkv, int row_stride, int k_off, int v_o
                                    const float *cos_table, const float *sin_table, const int *positions,
                                    const int *slot_mapping, int tokens, int num_q_heads, int num_kv_heads,
                                    int head_dim, int value_dim, int rot, int interleaved, float unit_eps,
-                                   int page_size, int dtype, hipStream_t stream) {
+                                   int page_size, int dtype, const void *bias, hipStream_t stream) {
     KVA_REQUIRE(tokens >= 0 && num_q_heads > 0 && num_kv_heads > 0 && value_dim > 0, "qk_encode_cache: bad sizes");
     KVA_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && head_dim <= ENC_MAX_HEAD_DIM,
                 "qk_encode_cache: head_dim %d must be even and at most %d", head_dim, ENC_MAX_HEAD_DIM);
@@ -185,7 +191,7 @@ extern "C" int kva_qk_encode_cache(void *qkv, int row_stride, int k_off, int v_o
     if (tokens == 0) return KVA_OK;
     if (rot == 0) cos_table = sin_table = reinterpret_cast<const float *>(qkv);     // never read
     const int vecs = head_dim / 8;
-    if (dtype == KVA_BF16 && interleaved && head_dim % 8 == 0 && (vecs & (vecs - 1)) == 0 && vecs <= KVA_WAVE &&
+    if (!bias && dtype == KVA_BF16 && interleaved && head_dim % 8 == 0 && (vecs & (vecs - 1)) == 0 && vecs <= KVA_WAVE &&
         row_stride % 8 == 0 && k_off % 8 == 0 && (reinterpret_cast<uintptr_t>(qkv) & 15) == 0) {
         hipLaunchKernelGGL(qk_encode_cache_vec_kernel, dim3(tokens), dim3(256), 0, stream, (bf16_t *)qkv, row_stride,
                            k_off, v_off, (bf16_t *)k_cache, (bf16_t *)v_cache, cos_table, sin_table, positions,
@@ -197,12 +203,12 @@ extern "C" int kva_qk_encode_cache(void *qkv, int row_stride, int k_off, int v_o
         hipLaunchKernelGGL(qk_encode_cache_kernel<float>, dim3(tokens), dim3(256), 0, stream, (float *)qkv, row_stride,
                            k_off, v_off, (float *)k_cache, (float *)v_cache, cos_table, sin_table, positions,
                            slot_mapping, num_q_heads, num_kv_heads, head_dim, value_dim, rot, interleaved, unit_eps,
-                           page_size);
+                           page_size, (const float *)bias);
     else if (dtype == KVA_BF16)
         hipLaunchKernelGGL(qk_encode_cache_kernel<bf16_t>, dim3(tokens), dim3(256), 0, stream, (bf16_t *)qkv,
                            row_stride, k_off, v_off, (bf16_t *)k_cache, (bf16_t *)v_cache, cos_table, sin_table,
                            positions, slot_mapping, num_q_heads, num_kv_heads, head_dim, value_dim, rot, interleaved,
-                           unit_eps, page_size);
+                           unit_eps, page_size, (const bf16_t *)bias);
     else KVA_REQUIRE(false, "qk_encode_cache: unsupported dtype %d", dtype);
     KVA_CHECK_LAUNCH("qk_encode_cache");
     return KVA_OK;

@@ -1,0 +1,298 @@
+// A routed feed-forward (mixture of experts) whose work stays on the device from the router's
+// logits to the weighted sum: no count of tokens per expert ever reaches the host, so the whole
+// layer can be captured into a graph.
+//
+//  * kva_moe_route:  scores = softmax(logits) over all router outputs; the `top` largest of
+//    scores + correction are chosen; their weights are the plain scores (optionally renormalised).
+//  * kva_moe_align:  the (token, choice) slots of real experts sorted by expert into a list padded
+//    so that every tile of 16 rows belongs to one expert (`sorted_slot`, -1 = padding), with the
+//    expert of every tile (`tile_expert`, -1 = unused tile).
+//  * kva_moe_expert_rows: one product per tile against its expert's matrix.  Mode 0 ("up"): rows of
+//    x gathered by slot / top, activation applied, written at the sorted position.  Mode 1 ("down"):
+//    rows at the sorted position, times the slot's routing weight, written at the slot (fp32).
+//    bf16 with K % 32 == 0 runs on the matrix cores, everything else (fp32 too) on a plain tiled
+//    kernel that adds k ascending.
+//  * kva_moe_combine: out[t] = sum over the token's choices of the slot's row, or, for a router
+//    output past the real experts (an identity expert), weight * x[t].
+//
+// A row's result depends on that row and its expert's matrix only, never on which other rows
+// share its tile: the same token gives the same numbers in any batch.
+#include "common.h"
+#include "attention_frag.h"
+#include <math.h>
+
+#define MOE_TILE 16
+#define MOE_MAX_EXPERTS 1024
+#define MOE_ROUTE_PER_LANE 8
+
+__device__ inline float moe_activate(float z, int act) {
+    if (act == 3) return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f));       // exact gelu
+    return kva_activate(z, act);
+}
+
+// ---- router ------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+moe_route_kernel(int *__restrict__ idx, float *__restrict__ wgt, const float *__restrict__ logits,
+                 const float *__restrict__ correction, int tokens, int outputs, int top, int renormalise) {
+    const int lane = threadIdx.x % KVA_WAVE;
+    const int t = blockIdx.x * (blockDim.x / KVA_WAVE) + threadIdx.x / KVA_WAVE;
+    if (t >= tokens) return;
+    float s[MOE_ROUTE_PER_LANE], ch[MOE_ROUTE_PER_LANE];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < MOE_ROUTE_PER_LANE; ++j) {
+        const int e = lane + j * KVA_WAVE;
+        s[j] = e < outputs ? logits[(size_t)t * outputs + e] : -INFINITY;
+        mx = fmaxf(mx, s[j]);
+    }
+    mx = wave_max(mx);
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < MOE_ROUTE_PER_LANE; ++j) {
+        const int e = lane + j * KVA_WAVE;
+        s[j] = e < outputs ? expf(s[j] - mx) : 0.f;
+        sum += s[j];
+    }
+    sum = wave_sum(sum);
+#pragma unroll
+    for (int j = 0; j < MOE_ROUTE_PER_LANE; ++j) {
+        const int e = lane + j * KVA_WAVE;
+        s[j] = s[j] / sum;
+        ch[j] = e < outputs ? s[j] + (correction ? correction[e] : 0.f) : -INFINITY;
+    }
+    float total = 0.f;
+    for (int k = 0; k < top; ++k) {
+        // the largest remaining choice score; of equal ones the lowest index
+        float bv = -INFINITY, bs = 0.f;
+        int be = 0x7fffffff;
+#pragma unroll
+        for (int j = 0; j < MOE_ROUTE_PER_LANE; ++j) {
+            const int e = lane + j * KVA_WAVE;
+            if (e < outputs && (ch[j] > bv || (ch[j] == bv && e < be))) { bv = ch[j]; be = e; bs = s[j]; }
+        }
+#pragma unroll
+        for (int off = KVA_WAVE / 2; off > 0; off >>= 1) {
+            const float ov = __shfl_xor(bv, off, KVA_WAVE), os = __shfl_xor(bs, off, KVA_WAVE);
+            const int oe = __shfl_xor(be, off, KVA_WAVE);
+            if (ov > bv || (ov == bv && oe < be)) { bv = ov; be = oe; bs = os; }
+        }
+#pragma unroll
+        for (int j = 0; j < MOE_ROUTE_PER_LANE; ++j)
+            if (lane + j * KVA_WAVE == be) ch[j] = -INFINITY;
+        total += bs;
+        if (lane == 0) {
+            idx[(size_t)t * top + k] = be;
+            wgt[(size_t)t * top + k] = bs;
+        }
+    }
+    if (renormalise && lane == 0)
+        for (int k = 0; k < top; ++k) wgt[(size_t)t * top + k] /= total;
+}
+
+extern "C" int kva_moe_route(int *idx, float *wgt, const float *logits, const float *correction, int tokens,
+                             int outputs, int top, int renormalise, hipStream_t stream) {
+    KVA_REQUIRE(idx && wgt && logits && tokens >= 0, "moe_route: missing operand");
+    KVA_REQUIRE(outputs > 0 && outputs <= KVA_WAVE * MOE_ROUTE_PER_LANE, "moe_route: %d router outputs (at most %d)",
+                outputs, KVA_WAVE * MOE_ROUTE_PER_LANE);
+    KVA_REQUIRE(top > 0 && top <= outputs, "moe_route: top %d of %d", top, outputs);
+    if (tokens == 0) return KVA_OK;
+    hipLaunchKernelGGL(moe_route_kernel, dim3((tokens + 3) / 4), dim3(256), 0, stream, idx, wgt, logits, correction,
+                       tokens, outputs, top, renormalise);
+    KVA_CHECK_LAUNCH("moe_route");
+    return KVA_OK;
+}
+
+// ---- slots sorted by expert --------------------------------------------------------------
+__global__ void __launch_bounds__(1024)
+moe_align_kernel(int *__restrict__ sorted_slot, int *__restrict__ tile_expert, const int *__restrict__ idx, int slots,
+                 int experts, int capacity, int max_tiles) {
+    __shared__ int count[MOE_MAX_EXPERTS], start[MOE_MAX_EXPERTS];
+    for (int e = threadIdx.x; e < experts; e += blockDim.x) count[e] = 0;
+    for (int p = threadIdx.x; p < capacity; p += blockDim.x) sorted_slot[p] = -1;
+    for (int i = threadIdx.x; i < max_tiles; i += blockDim.x) tile_expert[i] = -1;
+    __syncthreads();
+    for (int s = threadIdx.x; s < slots; s += blockDim.x) {
+        const int e = idx[s];
+        if (e >= 0 && e < experts) atomicAdd(&count[e], 1);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int at = 0;
+        for (int e = 0; e < experts; ++e) {
+            start[e] = at;
+            const int tiles = (count[e] + MOE_TILE - 1) / MOE_TILE;
+            for (int i = 0; i < tiles; ++i) tile_expert[at / MOE_TILE + i] = e;
+            at += tiles * MOE_TILE;
+            count[e] = 0;               // from here on: the next free place of the expert's run
+        }
+    }
+    __syncthreads();
+    for (int s = threadIdx.x; s < slots; s += blockDim.x) {
+        const int e = idx[s];
+        if (e >= 0 && e < experts) sorted_slot[start[e] + atomicAdd(&count[e], 1)] = s;
+    }
+}
+
+extern "C" int kva_moe_align(int *sorted_slot, int *tile_expert, const int *idx, int slots, int experts, int capacity,
+                             int max_tiles, hipStream_t stream) {
+    KVA_REQUIRE(sorted_slot && tile_expert && idx, "moe_align: missing operand");
+    KVA_REQUIRE(experts > 0 && experts <= MOE_MAX_EXPERTS, "moe_align: %d experts (at most %d)", experts, MOE_MAX_EXPERTS);
+    KVA_REQUIRE(capacity == max_tiles * MOE_TILE && capacity >= slots + experts * (MOE_TILE - 1),
+                "moe_align: a list of %d places cannot hold %d slots of %d experts in tiles of %d", capacity, slots,
+                experts, MOE_TILE);
+    hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(1024), 0, stream, sorted_slot, tile_expert, idx, slots, experts,
+                       capacity, max_tiles);
+    KVA_CHECK_LAUNCH("moe_align");
+    return KVA_OK;
+}
+
+// ---- one product per tile ------------------------------------------------------------------
+struct MoeRows {
+    const int *sorted_slot, *tile_expert;
+    const float *slot_weight;       // mode 1
+    int top, N, K, mode, act;
+};
+
+__device__ inline void moe_store(const MoeRows &a, void *out, int out_dtype, int place, int slot, int n, float v) {
+    if (a.mode == 0) {
+        v = moe_activate(v, a.act);
+        if (out_dtype == KVA_BF16) reinterpret_cast<uint16_t *>(out)[(size_t)place * a.N + n] = float_to_bf16_bits(v);
+        else reinterpret_cast<float *>(out)[(size_t)place * a.N + n] = v;
+    } else {
+        reinterpret_cast<float *>(out)[(size_t)slot * a.N + n] = v * a.slot_weight[slot];
+    }
+}
+
+// plain: a workgroup takes a tile of 16 rows and 64 outputs; thread (row, cx) 4 outputs
+template <typename T>
+__global__ void __launch_bounds__(256)
+moe_expert_rows_kernel(MoeRows a, void *__restrict__ out, int out_dtype, const T *__restrict__ x,
+                       const T *__restrict__ w) {
+    __shared__ float xs[MOE_TILE][33], ws[64][33];
+    const int tile = blockIdx.y, e = a.tile_expert[tile];
+    if (e < 0) return;
+    const int n0 = blockIdx.x * 64, row = threadIdx.x / 16, cx = threadIdx.x % 16;
+    const int place = tile * MOE_TILE + row, slot = a.sorted_slot[place];
+    const T *wm = w + (size_t)e * a.N * a.K;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int k0 = 0; k0 < a.K; k0 += 32) {
+        __syncthreads();
+        for (int i = threadIdx.x; i < MOE_TILE * 32; i += 256) {
+            const int rr = i / 32, kk = k0 + i % 32;
+            const int sl = a.sorted_slot[tile * MOE_TILE + rr];
+            const size_t src = a.mode == 0 ? (size_t)(sl < 0 ? 0 : sl / a.top) : (size_t)(tile * MOE_TILE + rr);
+            xs[rr][i % 32] = (kk < a.K && sl >= 0) ? to_float(x[src * a.K + kk]) : 0.f;
+        }
+        for (int i = threadIdx.x; i < 64 * 32; i += 256) {
+            const int nn = n0 + i / 32, kk = k0 + i % 32;
+            ws[i / 32][i % 32] = (nn < a.N && kk < a.K) ? to_float(wm[(size_t)nn * a.K + kk]) : 0.f;
+        }
+        __syncthreads();
+        for (int kk = 0; kk < 32; ++kk) {
+            const float xv = xs[row][kk];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[j] += xv * ws[cx + 16 * j][kk];
+        }
+    }
+    if (slot < 0) return;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int n = n0 + cx + 16 * j;
+        if (n < a.N) moe_store(a, out, out_dtype, place, slot, n, acc[j]);
+    }
+}
+
+// matrix cores: a wavefront takes a tile of 16 rows and NT tiles of 16 outputs; out^T[n, t] =
+// W[e][n, :] . x[t, :]; operands straight from memory, 16 bytes a lane and product
+template <int NT>
+__global__ void __launch_bounds__(256)
+moe_expert_rows_mfma_kernel(MoeRows a, void *__restrict__ out, int out_dtype, const bf16_t *__restrict__ x,
+                            const bf16_t *__restrict__ w) {
+    const int tile = blockIdx.y, e = a.tile_expert[tile];
+    if (e < 0) return;
+    const int lane = threadIdx.x % KVA_WAVE, wave = threadIdx.x / KVA_WAVE, r = lane & 15, g = lane >> 4;
+    const int n_first = (blockIdx.x * (blockDim.x / KVA_WAVE) + wave) * 16 * NT;
+    if (n_first >= a.N) return;
+    const int place = tile * MOE_TILE + r, slot = a.sorted_slot[place];
+    const size_t src = a.mode == 0 ? (size_t)(slot < 0 ? 0 : slot / a.top) : (size_t)place;
+    const bf16_t *xrow = x + src * a.K + 8 * g;
+    const bf16_t *wrow[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+        wrow[nt] = w + ((size_t)e * a.N + min(n_first + 16 * nt + r, a.N - 1)) * a.K + 8 * g;
+    f32x4 acc[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) acc[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int k0 = 0; k0 < a.K; k0 += 32) {
+        Frag8 xf, wf[NT];
+        xf.u4 = *reinterpret_cast<const uint4 *>(xrow + k0);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) wf[nt].u4 = *reinterpret_cast<const uint4 *>(wrow[nt] + k0);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[nt].v, xf.v, acc[nt], 0, 0, 0);
+    }
+    if (slot < 0) return;
+    // lane (row r, group g) holds outputs n0 + 4 g .. + 3 of its row
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int n = n_first + 16 * nt + 4 * g + i;
+            if (n < a.N) moe_store(a, out, out_dtype, place, slot, n, acc[nt][i]);
+        }
+}
+
+extern "C" int kva_moe_expert_rows(void *out, int out_dtype, const void *x, const void *w, int dtype,
+                                   const int *sorted_slot, const int *tile_expert, const float *slot_weight,
+                                   int max_tiles, int top, int N, int K, int mode, int act, hipStream_t stream) {
+    KVA_REQUIRE(out && x && w && sorted_slot && tile_expert, "moe_expert_rows: missing operand");
+    KVA_REQUIRE(mode == 0 || (mode == 1 && slot_weight && out_dtype == KVA_F32),
+                "moe_expert_rows: mode 1 writes fp32 rows times a weight per slot");
+    KVA_REQUIRE(mode == 1 || out_dtype == dtype, "moe_expert_rows: mode 0 writes rows of the operands' type");
+    KVA_REQUIRE(N > 0 && K > 0 && top > 0 && act >= 0 && act <= 3, "moe_expert_rows: bad sizes or activation");
+    KVA_REQUIRE(max_tiles >= 0 && max_tiles <= 65535, "moe_expert_rows: %d tiles are too many for one launch", max_tiles);
+    if (max_tiles == 0) return KVA_OK;
+    MoeRows a{sorted_slot, tile_expert, slot_weight, top, N, K, mode, act};
+    if (dtype == KVA_BF16 && K % 32 == 0) {
+        const int per_block = 4 * 16 * 4;
+        hipLaunchKernelGGL(moe_expert_rows_mfma_kernel<4>, dim3((N + per_block - 1) / per_block, max_tiles), dim3(256), 0,
+                           stream, a, out, out_dtype, (const bf16_t *)x, (const bf16_t *)w);
+    } else if (dtype == KVA_BF16) {
+        hipLaunchKernelGGL(moe_expert_rows_kernel<bf16_t>, dim3((N + 63) / 64, max_tiles), dim3(256), 0, stream, a, out,
+                           out_dtype, (const bf16_t *)x, (const bf16_t *)w);
+    } else if (dtype == KVA_F32) {
+        hipLaunchKernelGGL(moe_expert_rows_kernel<float>, dim3((N + 63) / 64, max_tiles), dim3(256), 0, stream, a, out,
+                           out_dtype, (const float *)x, (const float *)w);
+    } else KVA_REQUIRE(false, "moe_expert_rows: unsupported dtype %d", dtype);
+    KVA_CHECK_LAUNCH("moe_expert_rows");
+    return KVA_OK;
+}
+
+// ---- weighted sum --------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+moe_combine_kernel(void *__restrict__ out, const void *__restrict__ x, int dtype, const float *__restrict__ rows,
+                   const int *__restrict__ idx, const float *__restrict__ wgt, int width, int top, int experts) {
+    const size_t t = blockIdx.x;
+    for (int j = threadIdx.x; j < width; j += blockDim.x) {
+        float acc = 0.f;
+        for (int k = 0; k < top; ++k) {
+            const size_t s = t * top + k;
+            if (idx[s] < experts) acc += rows[s * width + j];
+            else acc += wgt[s] * (dtype == KVA_BF16 ? bf16_bits_to_float(reinterpret_cast<const uint16_t *>(x)[t * width + j])
+                                                    : reinterpret_cast<const float *>(x)[t * width + j]);
+        }
+        if (dtype == KVA_BF16) reinterpret_cast<uint16_t *>(out)[t * width + j] = float_to_bf16_bits(acc);
+        else reinterpret_cast<float *>(out)[t * width + j] = acc;
+    }
+}
+
+extern "C" int kva_moe_combine(void *out, const void *x, int dtype, const float *rows, const int *idx,
+                               const float *wgt, int tokens, int width, int top, int experts, hipStream_t stream) {
+    KVA_REQUIRE(out && x && rows && idx && wgt && width > 0 && top > 0, "moe_combine: missing operand");
+    KVA_REQUIRE(dtype == KVA_BF16 || dtype == KVA_F32, "moe_combine: unsupported dtype %d", dtype);
+    if (tokens <= 0) return KVA_OK;
+    hipLaunchKernelGGL(moe_combine_kernel, dim3(tokens), dim3(256), 0, stream, out, x, dtype, rows, idx, wgt, width, top,
+                       experts);
+    KVA_CHECK_LAUNCH("moe_combine");
+    return KVA_OK;
+}

@@ -1,0 +1,349 @@
+// Mixers that carry a fixed-size state per request instead of keys and values:
+//
+//  * kva_causal_conv_act / kva_conv_state_update: a short causal convolution over time per channel
+//    followed by silu; the last taps - 1 inputs of a request are part of its state.
+//  * kva_gated_delta_rule: per head S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q with
+//    unit-norm q and k, one decay g = exp(-exp(A_log) softplus(a + dt_bias)) per head and token.
+//  * kva_gated_linear_attention: per head S <- diag(alpha) S + k v^T; o = S^T q with a decay per
+//    key channel, alpha = sigmoid(z)^(1 / tau).
+//  * kva_head_norm_gate: every head of a row divided by its root mean square (optional) times a
+//    weight, times act(gate), times a constant, into a column range of a wider buffer.
+//
+// The state S [key channels, value channels] of a (request, head) is fp32 and lives in the seat's
+// state row between steps.  A wavefront takes 16 value columns of one head: lane = 16 * r + c owns
+// the rows i = r, r + 4, ... of column c, kept in LDS while the step's tokens of the request are
+// walked in order; sums over rows are finished between the four lanes of a column.  Columns are
+// independent of each other in both recurrences, so a head's columns go to different wavefronts.
+// The order of every sum depends on the sizes alone: a token's result is the same bit for bit
+// however the request's tokens were cut into steps and whatever else the step holds.
+#include "common.h"
+#include <math.h>
+
+#define REC_COLS 16          // value columns a wavefront takes
+#define REC_ROWGROUPS 4      // lanes that share a column
+#define REC_MAX_DIM 512
+
+__device__ inline float rec_ld(const void *p, int dtype, size_t i) {
+    return dtype == KVA_BF16 ? bf16_bits_to_float(reinterpret_cast<const uint16_t *>(p)[i])
+                             : reinterpret_cast<const float *>(p)[i];
+}
+
+__device__ inline void rec_st(void *p, int dtype, size_t i, float v) {
+    if (dtype == KVA_BF16) reinterpret_cast<uint16_t *>(p)[i] = float_to_bf16_bits(v);
+    else reinterpret_cast<float *>(p)[i] = v;
+}
+
+__device__ inline float rec_sigmoid(float z) { return 1.f / (1.f + expf(-z)); }
+__device__ inline float rec_silu(float z) { return z / (1.f + expf(-z)); }
+__device__ inline float rec_softplus(float z) { return fmaxf(z, 0.f) + log1pf(expf(-fabsf(z))); }
+
+// sum over the lanes that share a column (lanes c, c + 16, c + 32, c + 48), all of them get it
+__device__ inline float rec_column_sum(float v) {
+    v += __shfl_xor(v, 16, KVA_WAVE);
+    v += __shfl_xor(v, 32, KVA_WAVE);
+    return v;
+}
+
+// ---- short causal convolution + silu -----------------------------------------------------
+// out[row, c] = silu(sum_j w[c, j] * in(row - taps + 1 + j)[c]); inputs before the step's first
+// token of the request come from the seat's state [channels, taps - 1] (slot taps - 2 newest).
+__global__ void __launch_bounds__(256)
+causal_conv_act_kernel(float *__restrict__ out, int out_stride, const void *__restrict__ y, int y_dtype, int y_stride,
+                       int col_off, const void *__restrict__ w, int w_dtype, const float *__restrict__ state,
+                       size_t seat_stride, int conv_off, const int *__restrict__ entry_q_start,
+                       const int *__restrict__ entry_seat, int channels, int taps, int tokens_per_block) {
+    const int e = blockIdx.y;
+    const int q0 = entry_q_start[e], n = entry_q_start[e + 1] - q0;
+    const int first = blockIdx.x * tokens_per_block;
+    if (first >= n) return;
+    const int last = min(n, first + tokens_per_block);
+    const float *st = state + (size_t)entry_seat[e] * seat_stride + conv_off;
+    for (int c = threadIdx.x; c < channels; c += blockDim.x) {
+        for (int i = first; i < last; ++i) {
+            float acc = 0.f;
+            for (int j = 0; j < taps; ++j) {
+                const int src = i - (taps - 1) + j;
+                const float x = src >= 0 ? rec_ld(y, y_dtype, (size_t)(q0 + src) * y_stride + col_off + c)
+                                         : st[(size_t)c * (taps - 1) + (taps - 1) + src];
+                acc += rec_ld(w, w_dtype, (size_t)c * taps + j) * x;
+            }
+            out[(size_t)(q0 + i) * out_stride + c] = rec_silu(acc);
+        }
+    }
+}
+
+// the seat's last taps - 1 inputs after this step; a thread owns a channel (reads all, then writes)
+__global__ void __launch_bounds__(256)
+conv_state_update_kernel(float *__restrict__ state, size_t seat_stride, int conv_off, const void *__restrict__ y,
+                         int y_dtype, int y_stride, int col_off, const int *__restrict__ entry_q_start,
+                         const int *__restrict__ entry_seat, int channels, int taps) {
+    const int e = blockIdx.y;
+    const int q0 = entry_q_start[e], n = entry_q_start[e + 1] - q0;
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= channels || n <= 0) return;
+    float *st = state + (size_t)entry_seat[e] * seat_stride + conv_off + (size_t)c * (taps - 1);
+    float keep[16];
+    for (int s = 0; s < taps - 1; ++s) {
+        const int src = n - (taps - 1) + s;
+        keep[s] = src >= 0 ? rec_ld(y, y_dtype, (size_t)(q0 + src) * y_stride + col_off + c) : st[s + n];
+    }
+    for (int s = 0; s < taps - 1; ++s) st[s] = keep[s];
+}
+
+extern "C" int kva_causal_conv_act(float *out, int out_stride, const void *y, int y_dtype, int y_stride, int col_off,
+                                   const void *w, int w_dtype, float *state, long long seat_stride, int conv_off,
+                                   const int *entry_q_start, const int *entry_seat, int entries, int max_q_len,
+                                   int channels, int taps, hipStream_t stream) {
+    KVA_REQUIRE(out && y && w && state && entry_q_start && entry_seat, "causal_conv_act: missing operand");
+    KVA_REQUIRE(channels > 0 && taps >= 1 && taps <= 17, "causal_conv_act: taps %d must lie in 1..17", taps);
+    KVA_REQUIRE(entries >= 0 && entries <= 65535 && max_q_len >= 0, "causal_conv_act: bad batch");
+    if (entries == 0 || max_q_len == 0) return KVA_OK;
+    const int per = 8;
+    hipLaunchKernelGGL(causal_conv_act_kernel, dim3((max_q_len + per - 1) / per, entries), dim3(256), 0, stream, out,
+                       out_stride, y, y_dtype, y_stride, col_off, w, w_dtype, state, (size_t)seat_stride, conv_off,
+                       entry_q_start, entry_seat, channels, taps, per);
+    KVA_CHECK_LAUNCH("causal_conv_act");
+    if (taps > 1) {
+        hipLaunchKernelGGL(conv_state_update_kernel, dim3((channels + 255) / 256, entries), dim3(256), 0, stream, state,
+                           (size_t)seat_stride, conv_off, y, y_dtype, y_stride, col_off, entry_q_start, entry_seat,
+                           channels, taps);
+        KVA_CHECK_LAUNCH("conv_state_update");
+    }
+    return KVA_OK;
+}
+
+// ---- the two recurrences -----------------------------------------------------------------
+// LDS: S [dim][16] fp32, then per chunk of tokens q [chunk][dim], k [chunk][dim], (alpha [chunk][dim]),
+// and per token two numbers.
+struct RecArgs {
+    float *out;                 // [T, heads * vdim] fp32
+    float *state;               // seat rows; this mixer's S [heads, dim, vdim] at state_off
+    size_t seat_stride;
+    int state_off;
+    const int *entry_q_start, *entry_seat;
+    int heads, kv_heads, dim, vdim, chunk;
+};
+
+// Gated delta rule.  q, k, v are the convolution's fp32 output rows [T, conv_stride]: q at
+// column 0 (kv_heads x dim), k behind it, v behind that (heads x vdim).  beta and the decay's input
+// are columns of the projection y.
+__global__ void __launch_bounds__(KVA_WAVE)
+gated_delta_rule_kernel(RecArgs a, const float *__restrict__ qkv, int conv_stride, const void *__restrict__ y,
+                        int y_dtype, int y_stride, int beta_off, int decay_off, const float *__restrict__ a_log,
+                        const float *__restrict__ dt_bias, float unit_eps) {
+    extern __shared__ float lds[];
+    const int lane = threadIdx.x, c = lane % REC_COLS, r = lane / REC_COLS;
+    const int slices = (a.vdim + REC_COLS - 1) / REC_COLS;
+    const int head = blockIdx.x / slices, col = (blockIdx.x % slices) * REC_COLS + c;
+    const int e = blockIdx.y;
+    const int q0 = a.entry_q_start[e], n = a.entry_q_start[e + 1] - q0;
+    if (n <= 0) return;
+    const int d = a.dim, dv = a.vdim, kvh = head / (a.heads / a.kv_heads);
+    const bool on = col < dv;
+    float *S = lds, *qs = S + d * REC_COLS, *ks = qs + a.chunk * d, *bs = ks + a.chunk * d, *gs = bs + a.chunk;
+    float *Sg = a.state + (size_t)a.entry_seat[e] * a.seat_stride + a.state_off + (size_t)head * d * dv;
+    for (int i = r; i < d; i += REC_ROWGROUPS) S[i * REC_COLS + c] = on ? Sg[(size_t)i * dv + col] : 0.f;
+    const int k_col = a.kv_heads * d, v_col = 2 * a.kv_heads * d;
+    const float rate = expf(a_log[head]), bias = dt_bias[head], q_mul = 1.0f / sqrtf((float)d);
+    for (int t0 = 0; t0 < n; t0 += a.chunk) {
+        const int m = min(a.chunk, n - t0);
+        __syncthreads();
+        for (int x = lane; x < m * d; x += KVA_WAVE) {
+            const size_t row = (size_t)(q0 + t0 + x / d) * conv_stride;
+            qs[x] = qkv[row + kvh * d + x % d];
+            ks[x] = qkv[row + k_col + kvh * d + x % d];
+        }
+        __syncthreads();
+        // unit vectors: token tt by the four lanes 4 tt .. 4 tt + 3 (chunk <= 16)
+        {
+            const int tt = lane / 4, part = lane % 4;
+            float sq = 0.f, sk = 0.f;
+            if (tt < m)
+                for (int i = part; i < d; i += 4) {
+                    sq += qs[tt * d + i] * qs[tt * d + i];
+                    sk += ks[tt * d + i] * ks[tt * d + i];
+                }
+            sq += __shfl_xor(sq, 1, KVA_WAVE); sq += __shfl_xor(sq, 2, KVA_WAVE);
+            sk += __shfl_xor(sk, 1, KVA_WAVE); sk += __shfl_xor(sk, 2, KVA_WAVE);
+            const float mq = q_mul / sqrtf(sq + unit_eps), mk = 1.0f / sqrtf(sk + unit_eps);
+            __syncthreads();
+            if (tt < m) {
+                for (int i = part; i < d; i += 4) {
+                    qs[tt * d + i] *= mq;
+                    ks[tt * d + i] *= mk;
+                }
+                if (part == 0) {
+                    const size_t yrow = (size_t)(q0 + t0 + tt) * y_stride;
+                    bs[tt] = rec_sigmoid(rec_ld(y, y_dtype, yrow + beta_off + head));
+                    gs[tt] = expf(-rate * rec_softplus(rec_ld(y, y_dtype, yrow + decay_off + head) + bias));
+                }
+            }
+        }
+        __syncthreads();
+        for (int tt = 0; tt < m; ++tt) {
+            const float *q = qs + tt * d, *k = ks + tt * d;
+            const float g = gs[tt], beta = bs[tt];
+            const size_t row = (size_t)(q0 + t0 + tt);
+            const float v = on ? qkv[row * conv_stride + v_col + head * dv + col] : 0.f;
+            float dot = 0.f;
+            for (int i = r; i < d; i += REC_ROWGROUPS) dot += S[i * REC_COLS + c] * k[i];
+            dot = rec_column_sum(dot);
+            const float u = beta * (v - g * dot);
+            float o = 0.f;
+            for (int i = r; i < d; i += REC_ROWGROUPS) {
+                const float s = g * S[i * REC_COLS + c] + k[i] * u;
+                S[i * REC_COLS + c] = s;
+                o += s * q[i];
+            }
+            o = rec_column_sum(o);
+            if (on && r == 0) a.out[row * a.heads * dv + head * dv + col] = o;
+        }
+    }
+    if (on)
+        for (int i = r; i < d; i += REC_ROWGROUPS) Sg[(size_t)i * dv + col] = S[i * REC_COLS + c];
+}
+
+// Gated linear attention.  q, k, v and the decay's input z are columns of y (heads x dim, heads x
+// dim, heads x vdim, heads x dim; z may live in another buffer); q is multiplied by q_mul.
+__global__ void __launch_bounds__(KVA_WAVE)
+gated_linear_attention_kernel(RecArgs a, const void *__restrict__ y, int y_dtype, int y_stride, int q_off, int k_off,
+                              int v_off, const void *__restrict__ z, int z_dtype, int z_stride, int z_off,
+                              const float *__restrict__ z_bias, float inv_tau, float q_mul) {
+    extern __shared__ float lds[];
+    const int lane = threadIdx.x, c = lane % REC_COLS, r = lane / REC_COLS;
+    const int slices = (a.vdim + REC_COLS - 1) / REC_COLS;
+    const int head = blockIdx.x / slices, col = (blockIdx.x % slices) * REC_COLS + c;
+    const int e = blockIdx.y;
+    const int q0 = a.entry_q_start[e], n = a.entry_q_start[e + 1] - q0;
+    if (n <= 0) return;
+    const int d = a.dim, dv = a.vdim;
+    const bool on = col < dv;
+    float *S = lds, *qs = S + d * REC_COLS, *ks = qs + a.chunk * d, *as = ks + a.chunk * d;
+    float *Sg = a.state + (size_t)a.entry_seat[e] * a.seat_stride + a.state_off + (size_t)head * d * dv;
+    for (int i = r; i < d; i += REC_ROWGROUPS) S[i * REC_COLS + c] = on ? Sg[(size_t)i * dv + col] : 0.f;
+    for (int t0 = 0; t0 < n; t0 += a.chunk) {
+        const int m = min(a.chunk, n - t0);
+        __syncthreads();
+        for (int x = lane; x < m * d; x += KVA_WAVE) {
+            const size_t row = (size_t)(q0 + t0 + x / d);
+            const int i = head * d + x % d;
+            qs[x] = rec_ld(y, y_dtype, row * y_stride + q_off + i) * q_mul;
+            ks[x] = rec_ld(y, y_dtype, row * y_stride + k_off + i);
+            const float zz = rec_ld(z, z_dtype, row * z_stride + z_off + i) + z_bias[i];
+            as[x] = expf(-rec_softplus(-zz) * inv_tau);            // sigmoid(z)^(1 / tau)
+        }
+        __syncthreads();
+        for (int tt = 0; tt < m; ++tt) {
+            const float *q = qs + tt * d, *k = ks + tt * d, *al = as + tt * d;
+            const size_t row = (size_t)(q0 + t0 + tt);
+            const float v = on ? rec_ld(y, y_dtype, row * y_stride + v_off + head * dv + col) : 0.f;
+            float o = 0.f;
+            for (int i = r; i < d; i += REC_ROWGROUPS) {
+                const float s = al[i] * S[i * REC_COLS + c] + k[i] * v;
+                S[i * REC_COLS + c] = s;
+                o += s * q[i];
+            }
+            o = rec_column_sum(o);
+            if (on && r == 0) a.out[row * a.heads * dv + head * dv + col] = o;
+        }
+    }
+    if (on)
+        for (int i = r; i < d; i += REC_ROWGROUPS) Sg[(size_t)i * dv + col] = S[i * REC_COLS + c];
+}
+
+static int rec_chunk(int dim, int arrays) {
+    // tokens staged at a time: 16 where the LDS has room for them beside the state, else 4
+    const size_t room = 60 * 1024;
+    for (int chunk = 16; chunk >= 4; chunk /= 4)
+        if (((size_t)dim * REC_COLS + (size_t)chunk * dim * arrays + 2 * chunk) * sizeof(float) <= room) return chunk;
+    return 0;
+}
+
+static int rec_check(const char *what, const void *out, const void *state, const int *q_start, const int *seat,
+                     int entries, int heads, int kv_heads, int dim, int vdim) {
+    KVA_REQUIRE(out && state && q_start && seat, "%s: missing operand", what);
+    KVA_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "%s: %d heads over %d key heads", what, heads, kv_heads);
+    KVA_REQUIRE(dim > 0 && dim <= REC_MAX_DIM && vdim > 0, "%s: key size %d must lie in 1..%d", what, dim, REC_MAX_DIM);
+    KVA_REQUIRE(entries >= 0 && entries <= 65535, "%s: %d entries", what, entries);
+    return KVA_OK;
+}
+
+extern "C" int kva_gated_delta_rule(float *out, float *state, long long seat_stride, int state_off, const float *qkv,
+                                    int conv_stride, const void *y, int y_dtype, int y_stride, int beta_off,
+                                    int decay_off, const float *a_log, const float *dt_bias, float unit_eps,
+                                    const int *entry_q_start, const int *entry_seat, int entries, int heads,
+                                    int kv_heads, int dim, int vdim, hipStream_t stream) {
+    if (int rc = rec_check("gated_delta_rule", out, state, entry_q_start, entry_seat, entries, heads, kv_heads, dim, vdim)) return rc;
+    KVA_REQUIRE(qkv && y && a_log && dt_bias, "gated_delta_rule: missing operand");
+    if (entries == 0) return KVA_OK;
+    const int chunk = rec_chunk(dim, 2);
+    KVA_REQUIRE(chunk > 0, "gated_delta_rule: key size %d does not fit the LDS", dim);
+    RecArgs a{out, state, (size_t)seat_stride, state_off, entry_q_start, entry_seat, heads, kv_heads, dim, vdim, chunk};
+    const size_t lds = ((size_t)dim * REC_COLS + (size_t)chunk * dim * 2 + 2 * chunk) * sizeof(float);
+    const int slices = (vdim + REC_COLS - 1) / REC_COLS;
+    hipLaunchKernelGGL(gated_delta_rule_kernel, dim3(heads * slices, entries), dim3(KVA_WAVE), lds, stream, a, qkv,
+                       conv_stride, y, y_dtype, y_stride, beta_off, decay_off, a_log, dt_bias, unit_eps);
+    KVA_CHECK_LAUNCH("gated_delta_rule");
+    return KVA_OK;
+}
+
+extern "C" int kva_gated_linear_attention(float *out, float *state, long long seat_stride, int state_off,
+                                          const void *y, int y_dtype, int y_stride, int q_off, int k_off, int v_off,
+                                          const void *z, int z_dtype, int z_stride, int z_off, const float *z_bias,
+                                          float tau, float q_mul, const int *entry_q_start, const int *entry_seat,
+                                          int entries, int heads, int dim, int vdim, hipStream_t stream) {
+    if (int rc = rec_check("gated_linear_attention", out, state, entry_q_start, entry_seat, entries, heads, heads, dim, vdim)) return rc;
+    KVA_REQUIRE(y && z && z_bias && tau > 0.f, "gated_linear_attention: missing operand or tau <= 0");
+    if (entries == 0) return KVA_OK;
+    const int chunk = rec_chunk(dim, 3);
+    KVA_REQUIRE(chunk > 0, "gated_linear_attention: key size %d does not fit the LDS", dim);
+    RecArgs a{out, state, (size_t)seat_stride, state_off, entry_q_start, entry_seat, heads, heads, dim, vdim, chunk};
+    const size_t lds = ((size_t)dim * REC_COLS + (size_t)chunk * dim * 3) * sizeof(float);
+    const int slices = (vdim + REC_COLS - 1) / REC_COLS;
+    hipLaunchKernelGGL(gated_linear_attention_kernel, dim3(heads * slices, entries), dim3(KVA_WAVE), lds, stream, a, y,
+                       y_dtype, y_stride, q_off, k_off, v_off, z, z_dtype, z_stride, z_off, z_bias, 1.0f / tau, q_mul);
+    KVA_CHECK_LAUNCH("gated_linear_attention");
+    return KVA_OK;
+}
+
+// ---- per-head norm and gate ----------------------------------------------------------------
+// out[t, out_off + h dv + j] = (x[t, h, j] / sqrt(mean_j x^2 + eps) * w[j], or x as it is without a
+// weight) * act(gate[t, gate_off + h dv + j]) * mul;  act: 0 silu, 1 sigmoid.  One wavefront a head.
+__global__ void __launch_bounds__(256)
+head_norm_gate_kernel(void *__restrict__ out, int out_dtype, int out_stride, int out_off, const void *__restrict__ x,
+                      int x_dtype, const float *__restrict__ w, float eps, const void *__restrict__ gate,
+                      int gate_dtype, int gate_stride, int gate_off, int heads, int dv, int act, float mul) {
+    const size_t t = blockIdx.x;
+    const int lane = threadIdx.x % KVA_WAVE, wave = threadIdx.x / KVA_WAVE, waves = blockDim.x / KVA_WAVE;
+    for (int h = wave; h < heads; h += waves) {
+        const size_t base = (t * heads + h) * dv;
+        float inv = 1.f;
+        if (w) {
+            float sq = 0.f;
+            for (int j = lane; j < dv; j += KVA_WAVE) {
+                const float v = rec_ld(x, x_dtype, base + j);
+                sq += v * v;
+            }
+            inv = 1.0f / sqrtf(wave_sum(sq) / (float)dv + eps);
+        }
+        for (int j = lane; j < dv; j += KVA_WAVE) {
+            float v = rec_ld(x, x_dtype, base + j);
+            if (w) v = v * inv * w[j];
+            const float g = rec_ld(gate, gate_dtype, t * gate_stride + gate_off + h * dv + j);
+            v *= (act == 1 ? rec_sigmoid(g) : rec_silu(g)) * mul;
+            rec_st(out, out_dtype, t * out_stride + out_off + h * dv + j, v);
+        }
+    }
+}
+
+extern "C" int kva_head_norm_gate(void *out, int out_dtype, int out_stride, int out_off, const void *x, int x_dtype,
+                                  const float *w, float eps, const void *gate, int gate_dtype, int gate_stride,
+                                  int gate_off, int rows, int heads, int dv, int act, float mul, hipStream_t stream) {
+    KVA_REQUIRE(out && x && gate && heads > 0 && dv > 0 && rows >= 0, "head_norm_gate: missing operand or bad sizes");
+    KVA_REQUIRE(act == 0 || act == 1, "head_norm_gate: activation %d is neither silu (0) nor sigmoid (1)", act);
+    if (rows == 0) return KVA_OK;
+    hipLaunchKernelGGL(head_norm_gate_kernel, dim3(rows), dim3(256), 0, stream, out, out_dtype, out_stride, out_off, x,
+                       x_dtype, w, eps, gate, gate_dtype, gate_stride, gate_off, heads, dv, act, mul);
+    KVA_CHECK_LAUNCH("head_norm_gate");
+    return KVA_OK;
+}

@@ -26,7 +26,7 @@ __global__ void __launch_bounds__(256)
 layernorm_kernel(void *__restrict__ out1, void *__restrict__ out2, int out_dtype, void *__restrict__ x, int x_dtype,
                  const void *__restrict__ d1, int d1_dtype, const void *__restrict__ d2, int d2_dtype,
                  const void *__restrict__ w1, const void *__restrict__ w2, int w_dtype,
-                 const int *__restrict__ row_idx, int width, float eps, int rms) {
+                 const int *__restrict__ row_idx, int width, float eps, int rms, float delta_scale) {
     extern __shared__ float row_s[];
     __shared__ float red_s[4];
     const int r = blockIdx.x;
@@ -34,8 +34,14 @@ layernorm_kernel(void *__restrict__ out1, void *__restrict__ out2, int out_dtype
     float sum = 0.f;
     for (int j = threadIdx.x; j < width; j += blockDim.x) {
         float v = ld_as_float(x, x_dtype, src + j);
-        if (d1) v += ld_as_float(d1, d1_dtype, src + j);
-        if (d2) v += ld_as_float(d2, d2_dtype, src + j);
+        if (delta_scale == 1.0f) {
+            if (d1) v += ld_as_float(d1, d1_dtype, src + j);
+            if (d2) v += ld_as_float(d2, d2_dtype, src + j);
+        } else if (d1 || d2) {
+            // the branch outputs are added up first, and their sum enters the stream times a constant
+            const float b = (d1 ? ld_as_float(d1, d1_dtype, src + j) : 0.f) + (d2 ? ld_as_float(d2, d2_dtype, src + j) : 0.f);
+            v += delta_scale * b;
+        }
         if ((d1 || d2) && !row_idx) {
             st_from_float(x, x_dtype, src + j, v);
             v = ld_as_float(x, x_dtype, src + j);       // what the stream holds from now on
@@ -64,13 +70,13 @@ layernorm_kernel(void *__restrict__ out1, void *__restrict__ out2, int out_dtype
 extern "C" int kva_layernorm(void *out1, void *out2, int out_dtype, void *x, int x_dtype, const void *d1,
                              int d1_dtype, const void *d2, int d2_dtype, const void *w1, const void *w2,
                              int w_dtype, const int *row_idx, int rows, int width, float eps, int rms,
-                             hipStream_t stream) {
+                             float delta_scale, hipStream_t stream) {
     KVA_REQUIRE(rows >= 0 && width > 0 && width <= 16000, "layernorm: width %d must lie in 1..16000", width);
     KVA_REQUIRE(out1 && x && w1 && (out2 == nullptr) == (w2 == nullptr), "layernorm: an output without its weight");
     KVA_REQUIRE(eps >= 0.f, "layernorm: negative eps");
     if (rows == 0) return KVA_OK;
     hipLaunchKernelGGL(layernorm_kernel, dim3(rows), dim3(256), (size_t)width * sizeof(float), stream, out1, out2,
-                       out_dtype, x, x_dtype, d1, d1_dtype, d2, d2_dtype, w1, w2, w_dtype, row_idx, width, eps, rms);
+                       out_dtype, x, x_dtype, d1, d1_dtype, d2, d2_dtype, w1, w2, w_dtype, row_idx, width, eps, rms, delta_scale);
     KVA_CHECK_LAUNCH("layernorm");
     return KVA_OK;
 }

@@ -9,6 +9,7 @@ import torch
 from .. import parts as _parts  # noqa: F401  (registers the built-in part kinds)
 from . import llama as _llama   # noqa: F401  (registers LlamaForCausalLM)
 from . import gadopel as _gadopel   # noqa: F401  (registers Gadopel)
+from . import radilix as _radilix   # noqa: F401  (registers Radilix)
 from ..config.registry import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, STREAM_OPS, architecture_for)
 from ..models.spec import LayerCall, ModelSpec, TensorSpec
 from ..ops import kernels as K
@@ -260,6 +261,8 @@ class Model:
             if call.before is not None:
                 if isinstance(delta, NormedRows):
                     raise TypeError("an operation between layers takes the stream, not rows prepared for a norm")
+                if getattr(delta, "scale", 1.0) != 1.0:
+                    raise TypeError("an operation between layers adds pending branch outputs as they are, not times a constant")
                 pending = () if delta is None else (tuple(delta) if isinstance(delta, (tuple, list)) else (delta,))
                 hidden, delta = self.stream_ops[call.before].forward(hidden, pending, first), None
             # the norm that reads the residual stream after this block

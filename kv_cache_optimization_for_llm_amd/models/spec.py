@@ -22,7 +22,7 @@ class TensorSpec:
     dtype unless stored in 32-bit), ``"vector"`` (same rule) or ``"table"`` (integers, int32).
     """
 
-    shape: Tuple[int, ...]
+    shape: Tuple[Optional[int], ...]
     init: str = "normal"
     role: str = "matrix"
 

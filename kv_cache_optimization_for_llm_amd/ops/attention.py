@@ -376,11 +376,13 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
     value_dim = head_dim if value_dim is None else int(value_dim)
     if window <= 0:
         keep_first = 0
+    # the queries may be the first columns of a wider buffer: rows lie ``stride`` elements apart
+    stride = qkv.stride(0)
     if keep_first > 0 or sinks is not None or value_dim != head_dim:
         if rope is not None or max_parts:
             raise K.KernelError("paged_attention: kept first positions, sinks and a value size of its own "
                                 "go with neither rotation inside the kernel nor partial results")
-        if qkv.dtype == torch.bfloat16 and qkv.shape[1] % 8 == 0 \
+        if qkv.dtype == torch.bfloat16 and stride % 8 == 0 \
                 and K.attention_rows_mfma_supported(head_dim, value_dim, kv.page_size):
             from .latent_attention import choose_ranges
             # prompt portions with enough rows to fill the chip: two row tiles an item share their loads
@@ -391,11 +393,11 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
             # (with a window most ranges of a long context hold no visible key: their wavefronts end at once)
             ranges, per = choose_ranges(item_entry.shape[0] * num_kv_heads, batch.max_context,
                                         window + keep_first if window > 0 else 0)
-            return K.attention_rows_mfma(qkv, qkv.shape[1], out, kv.k_cache, kv.v_cache, kv.block_table, item_entry,
+            return K.attention_rows_mfma(qkv, stride, out, kv.k_cache, kv.v_cache, kv.block_table, item_entry,
                                          item_row0, batch.entry_seat, batch.entry_q_start, batch.entry_start_pos,
                                          num_q_heads, num_kv_heads, head_dim, scale, window, keep_first, sinks,
                                          value_dim, ranges, per, tiles)
-        return K.attention_rowwise(qkv, qkv.shape[1], out, kv.k_cache, kv.v_cache, kv.block_table,
+        return K.attention_rowwise(qkv, stride, out, kv.k_cache, kv.v_cache, kv.block_table,
                                    batch.tok_seat, batch.positions, num_q_heads, num_kv_heads,
                                    head_dim, scale, window, keep_first, sinks, value_dim)
     if rope is not None:
@@ -408,12 +410,11 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
                                      num_kv_heads, head_dim, scale, rope[0], rope[1],
                                      kv.slot_mapping if kv.writes else None, window, splits, per, keep_cached, waves)
     if not (qkv.dtype == torch.bfloat16 and K.attention_mfma_supported(head_dim, kv.page_size)
-            and qkv.shape[1] % 8 == 0):
-        return K.attention_rowwise(qkv, qkv.shape[1], out, kv.k_cache, kv.v_cache, kv.block_table,
+            and stride % 8 == 0):
+        return K.attention_rowwise(qkv, stride, out, kv.k_cache, kv.v_cache, kv.block_table,
                                    batch.tok_seat, batch.positions, num_q_heads, num_kv_heads,
                                    head_dim, scale, window)
     plan = _plan_for(batch, kv, num_q_heads, num_kv_heads, head_dim, max_parts)
-    stride = qkv.shape[1]
     for launch in plan:
         if launch[0] == "wave":
             _, (item_entry, item_row0, meta), tiles, splits, per, pair, covers_all, keep_cached, waves = launch

@@ -518,10 +518,11 @@ def attention_rows_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k
 
 def layernorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor, deltas=(),
               row_idx: Optional[torch.Tensor] = None, weight2: Optional[torch.Tensor] = None,
-              out2: Optional[torch.Tensor] = None, rms: bool = False) -> torch.Tensor:
+              out2: Optional[torch.Tensor] = None, rms: bool = False, delta_scale: float = 1.0) -> torch.Tensor:
     """``out = (x - mean) / sqrt(var + eps) * weight`` per row (``rms``: without taking the mean
     off).  ``deltas`` (up to two tensors of x's shape, any of the two storage types) are added to
-    ``x`` first, in place (not written back when ``row_idx`` gathers rows).  ``weight2`` / ``out2``:
+    ``x`` first, in place (not written back when ``row_idx`` gathers rows); with a ``delta_scale``
+    other than 1 their sum is multiplied by it before it enters ``x``.  ``weight2`` / ``out2``:
     a second normalised copy with another weight from the same statistics.  ``x`` may be fp32
     while ``out`` is bf16."""
     width = x.shape[-1]
@@ -544,7 +545,8 @@ def layernorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tens
         _opt(d1, "delta"), dtype_code(d1.dtype) if d1 is not None else 0,
         _opt(d2, "delta"), dtype_code(d2.dtype) if d2 is not None else 0,
         _dev(weight, "weight"), _opt(weight2, "weight2"), dtype_code(weight.dtype),
-        _opt(row_idx, "row_idx", torch.int32), rows, width, float(eps), 1 if rms else 0, _stream()), "layernorm")
+        _opt(row_idx, "row_idx", torch.int32), rows, width, float(eps), 1 if rms else 0, float(delta_scale),
+        _stream()), "layernorm")
     return out
 
 
@@ -597,16 +599,22 @@ def head_gate(x: torch.Tensor, gates: torch.Tensor, heads: int) -> torch.Tensor:
 def qk_encode_cache(qkv: torch.Tensor, positions: torch.Tensor, num_q_heads: int, num_kv_heads: int, head_dim: int,
                     value_dim: int, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], interleaved: bool,
                     unit_eps: Optional[float], k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
-                    slot_mapping: Optional[torch.Tensor]) -> None:
+                    slot_mapping: Optional[torch.Tensor], bias: Optional[torch.Tensor] = None) -> None:
     """Rotates the first ``2 * cos.shape[1]`` elements of every Q and K head of ``qkv``
     ``[T, nq d + nkv d + nkv value_dim]`` (pair i = elements (2i, 2i + 1) when ``interleaved``, else
     (i, i + rot / 2)), then - with ``unit_eps`` - divides every head by its root mean square; Q in
-    place, K and the plain V into the paged cache at ``slot_mapping``."""
+    place, K and the plain V into the paged cache at ``slot_mapping``.  ``qkv`` may be the first
+    columns of a wider buffer (rows ``qkv.stride(0)`` apart).  ``bias`` (qkv's type, one value per
+    column) is added to Q, K and V first: the projection's bias, applied here."""
     tokens = qkv.shape[0]
     k_off = num_q_heads * head_dim
     v_off = k_off + num_kv_heads * head_dim
-    if qkv.dim() != 2 or qkv.shape[1] != v_off + num_kv_heads * value_dim or positions.shape != (tokens,):
+    if qkv.dim() != 2 or qkv.shape[1] != v_off + num_kv_heads * value_dim or positions.shape != (tokens,) \
+            or qkv.stride(1) != 1:
         raise KernelError(f"qk_encode_cache: qkv {tuple(qkv.shape)} is not [T, nq d + nkv d + nkv dv]")
+    if bias is not None and (bias.shape != (qkv.shape[1],) or bias.dtype != qkv.dtype):
+        raise KernelError("qk_encode_cache: the bias has one value of qkv's type per column")
+    row_stride = qkv.stride(0) if tokens > 1 else qkv.shape[1]
     rot = 0
     if cos is not None:
         if sin is None or cos.shape != sin.shape or cos.dim() != 2:
@@ -620,11 +628,11 @@ def qk_encode_cache(qkv: torch.Tensor, positions: torch.Tensor, num_q_heads: int
             raise KernelError("qk_encode_cache: K and V cache of qkv's dtype and one slot per token are needed")
         page_size = check_kv_cache_shapes("qk_encode_cache", k_cache, v_cache, num_kv_heads, head_dim, value_dim)
     check(hip_lib().kva_qk_encode_cache(
-        _dev(qkv, "qkv"), qkv.shape[1], k_off, v_off, _opt(k_cache, "k_cache"), _opt(v_cache, "v_cache"),
+        _dev(qkv, "qkv", contiguous=False), row_stride, k_off, v_off, _opt(k_cache, "k_cache"), _opt(v_cache, "v_cache"),
         _opt(cos, "cos", torch.float32), _opt(sin, "sin", torch.float32), _dev(positions, "positions", torch.int32),
         _opt(slot_mapping if write else None, "slot_mapping", torch.int32), tokens, num_q_heads, num_kv_heads,
         head_dim, value_dim, rot, 1 if interleaved else 0, -1.0 if unit_eps is None else float(unit_eps),
-        page_size, dtype_code(qkv.dtype), _stream()), "qk_encode_cache")
+        page_size, dtype_code(qkv.dtype), _opt(bias, "bias"), _stream()), "qk_encode_cache")
 
 
 def latent_encode_cache(y: torch.Tensor, kv_off: int, q_lat: torch.Tensor, cache: Optional[torch.Tensor],
@@ -1354,6 +1362,205 @@ def normed_rows_finish(scaled: torch.Tensor, sumsq: torch.Tensor, norm_width: in
 
 
 # --------------------------------------------------------------------------------------
+# Mixers with a fixed-size state per request, and what goes with them.
+def _entries(batch_arrays, what: str):
+    q_start, seat = batch_arrays
+    entries = seat.shape[0]
+    if q_start.shape != (entries + 1,):
+        raise KernelError(f"{what}: entries + 1 starts, one seat per entry")
+    return _dev(q_start, "entry_q_start", torch.int32), _dev(seat, "entry_seat", torch.int32), entries
+
+
+def _state_row(state: torch.Tensor, offset: int, elements: int, what: str) -> int:
+    if state.dim() != 2 or state.dtype != torch.float32 or not state.is_contiguous() \
+            or offset < 0 or offset + elements > state.shape[1]:
+        raise KernelError(f"{what}: the state is fp32 [seats, n] and holds {elements} elements from {offset} on")
+    return state.shape[1]
+
+
+def causal_conv_act(y: torch.Tensor, col_off: int, weight: torch.Tensor, out: torch.Tensor, state: torch.Tensor,
+                    state_off: int, entry_q_start: torch.Tensor, entry_seat: torch.Tensor, max_q_len: int) -> torch.Tensor:
+    """A short causal convolution over time per channel, then silu: ``out[t, c] = silu(sum_j
+    weight[c, j] * in[t - taps + 1 + j, c])`` with ``in`` the columns ``col_off ..`` of ``y``; the inputs
+    before an entry's first token come from the seat's state (``taps - 1`` values per channel at
+    ``state_off``, oldest first; zero for a fresh seat), which afterwards holds the entry's last ones.
+    ``out`` is fp32 ``[T, channels]``."""
+    tokens, channels = out.shape
+    if weight.dim() != 2 or weight.shape[0] != channels or out.dtype != torch.float32 or y.dim() != 2 \
+            or y.shape[0] != tokens or col_off < 0 or col_off + channels > y.shape[1]:
+        raise KernelError(f"causal_conv_act: y {tuple(y.shape)}, weight {tuple(weight.shape)}, out {tuple(out.shape)} do not fit")
+    taps = weight.shape[1]
+    seat_stride = _state_row(state, state_off, channels * (taps - 1), "causal_conv_act")
+    qs, seat, entries = _entries((entry_q_start, entry_seat), "causal_conv_act")
+    check(hip_lib().kva_causal_conv_act(
+        _dev(out, "out"), channels, _dev(y, "y"), dtype_code(y.dtype), y.shape[1], int(col_off), _dev(weight, "weight"),
+        dtype_code(weight.dtype), _dev(state, "state"), seat_stride, int(state_off), qs, seat, entries, int(max_q_len),
+        channels, taps, _stream()), "causal_conv_act")
+    return out
+
+
+def gated_delta_rule(qkv: torch.Tensor, y: torch.Tensor, beta_off: int, decay_off: int, a_log: torch.Tensor,
+                     dt_bias: torch.Tensor, out: torch.Tensor, state: torch.Tensor, state_off: int,
+                     entry_q_start: torch.Tensor, entry_seat: torch.Tensor, heads: int, kv_heads: int, dim: int,
+                     vdim: int, unit_eps: float = 1e-6) -> torch.Tensor:
+    """Per head and token, in order: ``S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q`` with
+    q and k made unit vectors (``x / sqrt(sum x^2 + unit_eps)``, q also times ``dim^-1/2``),
+    ``beta = sigmoid(y[t, beta_off + h])`` and ``g = exp(-exp(a_log[h]) softplus(y[t, decay_off + h] +
+    dt_bias[h]))``.  ``qkv`` fp32 ``[T, 2 kv_heads dim + heads vdim]`` holds q, k (``kv_heads`` heads) and v;
+    head h uses q/k head ``h // (heads / kv_heads)``.  ``S`` ``[heads, dim, vdim]`` lives at ``state_off`` of
+    the seat's fp32 state row.  ``out`` fp32 ``[T, heads * vdim]``."""
+    tokens = out.shape[0]
+    if qkv.shape != (tokens, 2 * kv_heads * dim + heads * vdim) or qkv.dtype != torch.float32 \
+            or out.shape != (tokens, heads * vdim) or out.dtype != torch.float32 or y.dim() != 2 or y.shape[0] != tokens:
+        raise KernelError(f"gated_delta_rule: qkv {tuple(qkv.shape)}, y {tuple(y.shape)}, out {tuple(out.shape)} do not fit")
+    if not (0 <= beta_off <= y.shape[1] - heads and 0 <= decay_off <= y.shape[1] - heads):
+        raise KernelError("gated_delta_rule: beta and decay columns lie outside y")
+    if a_log.shape != (heads,) or dt_bias.shape != (heads,):
+        raise KernelError("gated_delta_rule: one rate and one bias per head")
+    seat_stride = _state_row(state, state_off, heads * dim * vdim, "gated_delta_rule")
+    qs, seat, entries = _entries((entry_q_start, entry_seat), "gated_delta_rule")
+    check(hip_lib().kva_gated_delta_rule(
+        _dev(out, "out"), _dev(state, "state"), seat_stride, int(state_off), _dev(qkv, "qkv"), qkv.shape[1],
+        _dev(y, "y"), dtype_code(y.dtype), y.shape[1], int(beta_off), int(decay_off),
+        _dev(a_log, "a_log", torch.float32), _dev(dt_bias, "dt_bias", torch.float32), float(unit_eps), qs, seat,
+        entries, heads, kv_heads, dim, vdim, _stream()), "gated_delta_rule")
+    return out
+
+
+def gated_linear_attention(y: torch.Tensor, q_off: int, k_off: int, v_off: int, z: torch.Tensor, z_bias: torch.Tensor,
+                           tau: float, q_mul: float, out: torch.Tensor, state: torch.Tensor, state_off: int,
+                           entry_q_start: torch.Tensor, entry_seat: torch.Tensor, heads: int, dim: int,
+                           vdim: int) -> torch.Tensor:
+    """Per head and token, in order: ``S <- diag(alpha) S + k v^T; o = S^T (q_mul q)`` with a decay
+    per key channel ``alpha = sigmoid(z + z_bias)^(1 / tau)``.  q, k (``heads x dim``) and v (``heads x
+    vdim``) are columns of ``y`` from ``q_off``, ``k_off``, ``v_off`` on; ``z`` is ``[T, heads * dim]``.
+    ``out`` fp32 ``[T, heads * vdim]``."""
+    tokens = out.shape[0]
+    if y.dim() != 2 or y.shape[0] != tokens or out.shape != (tokens, heads * vdim) or out.dtype != torch.float32 \
+            or z.shape != (tokens, heads * dim) or z_bias.shape != (heads * dim,):
+        raise KernelError(f"gated_linear_attention: y {tuple(y.shape)}, z {tuple(z.shape)}, out {tuple(out.shape)} do not fit")
+    for off, n in ((q_off, heads * dim), (k_off, heads * dim), (v_off, heads * vdim)):
+        if not 0 <= off <= y.shape[1] - n:
+            raise KernelError("gated_linear_attention: q, k or v columns lie outside y")
+    seat_stride = _state_row(state, state_off, heads * dim * vdim, "gated_linear_attention")
+    qs, seat, entries = _entries((entry_q_start, entry_seat), "gated_linear_attention")
+    check(hip_lib().kva_gated_linear_attention(
+        _dev(out, "out"), _dev(state, "state"), seat_stride, int(state_off), _dev(y, "y"), dtype_code(y.dtype),
+        y.shape[1], int(q_off), int(k_off), int(v_off), _dev(z, "z"), dtype_code(z.dtype), z.shape[1], 0,
+        _dev(z_bias, "z_bias", torch.float32), float(tau), float(q_mul), qs, seat, entries, heads, dim, vdim,
+        _stream()), "gated_linear_attention")
+    return out
+
+
+HEAD_GATES = {"silu": 0, "sigmoid": 1}
+
+
+def head_norm_gate(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, gate: torch.Tensor, gate_off: int,
+                   out: torch.Tensor, out_off: int, heads: int, vdim: int, activation: str, mul: float = 1.0) -> torch.Tensor:
+    """``out[t, out_off + h vdim + j] = n(x)[t, h, j] * act(gate[t, gate_off + h vdim + j]) * mul`` where
+    ``n`` divides every head by its root mean square (``sqrt(mean_j x^2 + eps)``) and multiplies by
+    ``weight[j]`` (fp32, shared by the heads), or leaves x as it is without a weight.  ``gate`` and
+    ``out`` may be wider buffers; ``act`` is silu or sigmoid."""
+    rows = x.shape[0]
+    if x.shape != (rows, heads * vdim) or gate.dim() != 2 or gate.shape[0] != rows or out.dim() != 2 \
+            or out.shape[0] != rows or not 0 <= gate_off <= gate.shape[1] - heads * vdim \
+            or not 0 <= out_off <= out.shape[1] - heads * vdim:
+        raise KernelError(f"head_norm_gate: x {tuple(x.shape)}, gate {tuple(gate.shape)}, out {tuple(out.shape)} do not fit")
+    if weight is not None and (weight.shape != (vdim,) or weight.dtype != torch.float32):
+        raise KernelError("head_norm_gate: the weight is fp32, one value per element of a head")
+    if activation not in HEAD_GATES:
+        raise KernelError(f"head_norm_gate: activation {activation!r} is not one of {sorted(HEAD_GATES)}")
+    check(hip_lib().kva_head_norm_gate(
+        _dev(out, "out"), dtype_code(out.dtype), out.shape[1], int(out_off), _dev(x, "x"), dtype_code(x.dtype),
+        _opt(weight, "weight"), float(eps), _dev(gate, "gate"), dtype_code(gate.dtype), gate.shape[1], int(gate_off),
+        rows, heads, vdim, HEAD_GATES[activation], float(mul), _stream()), "head_norm_gate")
+    return out
+
+
+# --------------------------------------------------------------------------------------
+# Routed experts.
+MOE_TILE = 16
+EXPERT_ACTIVATIONS = {"silu": 0, "relu": 1, "gelu_tanh": 2, "gelu": 3}
+
+
+def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int, idx: torch.Tensor,
+              wgt: torch.Tensor, renormalise: bool = False) -> None:
+    """``scores = softmax(logits)`` over all router outputs; the ``top`` largest of ``scores +
+    correction`` are chosen (of equal ones the lowest index) into ``idx`` ``[T, top]``; ``wgt`` gets their
+    plain scores, divided by their sum with ``renormalise``."""
+    tokens, outputs = logits.shape
+    if logits.dtype != torch.float32 or idx.shape != (tokens, top) or wgt.shape != (tokens, top) \
+            or (correction is not None and correction.shape != (outputs,)):
+        raise KernelError(f"moe_route: logits {tuple(logits.shape)}, idx {tuple(idx.shape)}, wgt {tuple(wgt.shape)} do not fit")
+    check(hip_lib().kva_moe_route(_dev(idx, "idx", torch.int32), _dev(wgt, "wgt", torch.float32), _dev(logits, "logits"),
+                                  _opt(correction, "correction", torch.float32), tokens, outputs, int(top),
+                                  1 if renormalise else 0, _stream()), "moe_route")
+
+
+def moe_tiles(slots: int, experts: int) -> int:
+    """Tiles of 16 rows that hold ``slots`` (token, choice) pairs sorted by expert, whatever the split."""
+    return (int(slots) + int(experts) * (MOE_TILE - 1) + MOE_TILE - 1) // MOE_TILE
+
+
+def moe_align(idx: torch.Tensor, experts: int, sorted_slot: torch.Tensor, tile_expert: torch.Tensor) -> None:
+    """The slots ``idx.view(-1)`` that name one of the first ``experts`` router outputs, sorted by
+    expert into ``sorted_slot`` (every tile of 16 places belongs to one expert, -1 pads) with the
+    tiles' experts in ``tile_expert`` (-1: unused)."""
+    slots, tiles = idx.numel(), tile_expert.shape[0]
+    if sorted_slot.shape != (tiles * MOE_TILE,) or tiles < moe_tiles(slots, experts):
+        raise KernelError(f"moe_align: {tiles} tiles cannot hold {slots} slots of {experts} experts")
+    check(hip_lib().kva_moe_align(_dev(sorted_slot, "sorted_slot", torch.int32), _dev(tile_expert, "tile_expert", torch.int32),
+                                  _dev(idx, "idx", torch.int32), slots, int(experts), tiles * MOE_TILE, tiles,
+                                  _stream()), "moe_align")
+
+
+def moe_expert_rows(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, sorted_slot: torch.Tensor,
+                    tile_expert: torch.Tensor, top: int, *, activation: Optional[str] = None,
+                    slot_weight: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One product per tile against its expert's matrix ``w[e]`` ``[N, K]``.  With an ``activation``
+    (the first product): row ``slot // top`` of ``x`` ``[T, K]``, activated, goes to the slot's sorted
+    place of ``out`` ``[places, N]`` (x's type).  With ``slot_weight`` (the second): the row at the
+    sorted place of ``x`` ``[places, K]``, times the slot's weight, goes to row ``slot`` of ``out`` fp32
+    ``[slots, N]``."""
+    tiles = tile_expert.shape[0]
+    if (activation is None) == (slot_weight is None):
+        raise KernelError("moe_expert_rows: either an activation (first product) or slot weights (second)")
+    if w.dim() != 3 or w.dtype != x.dtype or x.dim() != 2 or x.shape[1] != w.shape[2] or out.dim() != 2 \
+            or out.shape[1] != w.shape[1] or sorted_slot.shape != (tiles * MOE_TILE,):
+        raise KernelError(f"moe_expert_rows: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
+    if activation is not None:
+        if activation not in EXPERT_ACTIVATIONS:
+            raise KernelError(f"moe_expert_rows: activation {activation!r} is not one of {sorted(EXPERT_ACTIVATIONS)}")
+        if out.shape[0] != tiles * MOE_TILE or out.dtype != x.dtype:
+            raise KernelError("moe_expert_rows: the first product writes one row of x's type per sorted place")
+    else:
+        if x.shape[0] != tiles * MOE_TILE or out.dtype != torch.float32 or slot_weight.numel() != out.shape[0] \
+                or slot_weight.dtype != torch.float32:
+            raise KernelError("moe_expert_rows: the second product reads sorted places and writes fp32 rows per slot")
+    check(hip_lib().kva_moe_expert_rows(
+        _dev(out, "out"), dtype_code(out.dtype), _dev(x, "x"), _dev(w, "w"), dtype_code(x.dtype),
+        _dev(sorted_slot, "sorted_slot", torch.int32), _dev(tile_expert, "tile_expert", torch.int32),
+        _opt(slot_weight, "slot_weight"), tiles, int(top), w.shape[1], w.shape[2], 0 if activation is not None else 1,
+        EXPERT_ACTIVATIONS.get(activation, 0), _stream()), "moe_expert_rows")
+    return out
+
+
+def moe_combine(x: torch.Tensor, rows: torch.Tensor, idx: torch.Tensor, wgt: torch.Tensor, experts: int,
+                out: torch.Tensor) -> torch.Tensor:
+    """``out[t] = sum over the token's choices`` of the slot's row of ``rows`` (fp32 ``[T * top, width]``,
+    already weighted) or, for a choice past the real ``experts`` (an identity expert), ``wgt * x[t]``."""
+    tokens, width = x.shape
+    top = idx.shape[1]
+    if out.shape != x.shape or out.dtype != x.dtype or rows.shape != (tokens * top, width) or rows.dtype != torch.float32 \
+            or idx.shape != (tokens, top) or wgt.shape != (tokens, top):
+        raise KernelError(f"moe_combine: x {tuple(x.shape)}, rows {tuple(rows.shape)}, idx {tuple(idx.shape)} do not fit")
+    check(hip_lib().kva_moe_combine(_dev(out, "out"), _dev(x, "x"), dtype_code(x.dtype), _dev(rows, "rows"),
+                                    _dev(idx, "idx", torch.int32), _dev(wgt, "wgt", torch.float32), tokens, width, top,
+                                    int(experts), _stream()), "moe_combine")
+    return out
+
+
+# --------------------------------------------------------------------------------------
 # Measurement: device time per class of kernel, from events around every launch.
 KERNEL_CLASSES = {
     "embed_gather": "embedding", "embed_gather_prep": "embedding", "rmsnorm": "norm", "normed_rows_finish": "norm",
@@ -1369,6 +1576,10 @@ KERNEL_CLASSES = {
     "gemm_skinny": "gemm (few rows)", "gemm_skinny_qkv_rope": "gemm (few rows)",
     "gemv": "gemm (few rows)", "gemv_qkv_rope": "gemm (few rows)", "gemv_merged": "gemm (few rows)",
     "sample": "sampling", "mark_tokens": "sampling",
+    "causal_conv_act": "recurrent mixers", "gated_delta_rule": "recurrent mixers",
+    "gated_linear_attention": "recurrent mixers", "head_norm_gate": "elementwise",
+    "moe_route": "routed experts", "moe_align": "routed experts", "moe_expert_rows": "routed experts",
+    "moe_combine": "routed experts",
 }
 
 

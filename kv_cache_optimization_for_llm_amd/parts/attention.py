@@ -19,7 +19,8 @@ from ..models.spec import PartSpec, TensorSpec
 from ..ops import attention as attn_ops
 from ..ops import kernels as K
 from ..ops.gemm_bf16 import SKINNY_MAX_ROWS
-from .base import BranchTail, KVCacheSpec, Mixer, MixerContext, NormedRows, attention_cache_spec
+from .base import (BranchTail, KVCacheSpec, Mixer, MixerContext, NormedRows, ProjectedMixer,
+                   attention_cache_spec)
 from .linear import Linear
 
 
@@ -176,3 +177,94 @@ class GQAAttention(Mixer):
             if fused is not None:
                 return fused
         return self.o(out)
+
+
+@MIXERS.register("gated_gqa_attention")
+class GatedGQAAttention(ProjectedMixer):
+    """Grouped-query causal attention over the paged cache with what :class:`GQAAttention` leaves
+    out: biases on the q, k and v projections (added where the heads are rotated and cached) and an
+    output gate - the concatenated heads times ``sigmoid(W_g x)``, element by element, before the
+    output projection.  The position encoding is a part like everywhere (a rotation of the first
+    elements of a head passes the rest unchanged); window, kept first positions and a value size of
+    its own are the options :func:`~..ops.attention.paged_attention` has.  As a
+    :class:`~.base.ProjectedMixer` it runs alone or beside other mixers on the same input."""
+
+    graph_safe = True
+
+    def __init__(self, prefix: str, *, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 scale: float, position: PartSpec, value_dim: Optional[int] = None, window: int = 0,
+                 keep_first: int = 0, bias: bool = False, gate: Optional[str] = "sigmoid",
+                 tensor_names: Optional[Dict[str, str]] = None):
+        """``bias``: q, k and v have biases named like their matrices with ``bias_suffix`` added.
+        ``gate``: ``"sigmoid"``, ``"silu"`` or ``None``.  ``tensor_names`` maps ``q k v g o`` and
+        ``bias_suffix`` to names behind ``prefix``."""
+        super().__init__(prefix)
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} heads is not a multiple of {num_kv_heads} kv heads")
+        if gate not in (None, "sigmoid", "silu"):
+            raise ValueError(f"output gate {gate!r} is not one of None, 'sigmoid', 'silu'")
+        self.hidden_size, self.num_heads, self.num_kv_heads = int(hidden_size), int(num_heads), int(num_kv_heads)
+        self.head_dim, self.scale, self.window = int(head_dim), float(scale), int(window)
+        self.keep_first = int(keep_first) if self.window > 0 else 0
+        self.value_dim = int(head_dim if value_dim is None else value_dim)
+        self.bias, self.gate = bool(bias), gate
+        names = dict(q="q", k="k", v="v", g="g", o="o", bias_suffix=".b")
+        names.update(tensor_names or {})
+        self.bias_suffix = names.pop("bias_suffix")
+        self.names = {key: prefix + name for key, name in names.items()}
+        self.position = POSITION_ENCODINGS.get(position.kind)(**position.params)
+        self.inner_width = self.num_heads * self.value_dim
+        self.qkv_width = (self.num_heads + self.num_kv_heads) * self.head_dim + self.num_kv_heads * self.value_dim
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        n, d, dv, W = self.names, self.head_dim, self.value_dim, self.hidden_size
+        specs = {n["q"]: TensorSpec((self.num_heads * d, W)), n["k"]: TensorSpec((self.num_kv_heads * d, W)),
+                 n["v"]: TensorSpec((self.num_kv_heads * dv, W)), n["o"]: TensorSpec((W, self.inner_width))}
+        if self.gate is not None:
+            specs[n["g"]] = TensorSpec((self.inner_width, W))
+        if self.bias:
+            for key in "qkv":
+                specs[n[key] + self.bias_suffix] = TensorSpec((specs[n[key]].shape[0],), init="normal", role="vector")
+        return specs
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        n = self.names
+        rows = [tensors[n[key]] for key in "qkv"] + ([tensors[n["g"]]] if self.gate is not None else [])
+        self._w_in = torch.cat(rows, dim=0).contiguous()
+        self._w_out = tensors[n["o"]]
+        self.qkv_bias = torch.cat([tensors[n[key] + self.bias_suffix] for key in "qkv"]).contiguous() if self.bias else None
+        self.load_projections()
+
+    def input_weight(self) -> torch.Tensor:
+        return self._w_in
+
+    def output_weight(self) -> torch.Tensor:
+        return self._w_out
+
+    def kv_cache_spec(self) -> KVCacheSpec:
+        return attention_cache_spec(self.num_kv_heads, self.head_dim, kind="window" if self.window > 0 else "full",
+                                    window=self.window, value_dim=self.value_dim, keep_first=self.keep_first)
+
+    def activation_elements(self) -> int:
+        return self.qkv_width + 3 * self.inner_width + self.hidden_size
+
+    def forward_inner(self, y, col0, ctx: MixerContext, state_off, out, out_col0, mul) -> None:
+        batch, kv = ctx.batch, ctx.kv
+        qkv = y[:, col0:col0 + self.qkv_width]
+        write = kv is not None and kv.writes
+        cos, sin = self.position.tables(y.device) if hasattr(self.position, "tables") else (None, None)
+        K.qk_encode_cache(qkv, batch.positions, self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim,
+                          cos, sin, getattr(self.position, "pairing", "half") == "interleaved",
+                          getattr(self.position, "unit_norm_eps", None),
+                          kv.k_cache if write else None, kv.v_cache if write else None,
+                          kv.slot_mapping if write else None, bias=self.qkv_bias)
+        direct = self.gate is None and mul == 1.0 and out_col0 == 0 and out.shape[1] == self.inner_width
+        heads = out if direct else torch.empty((y.shape[0], self.inner_width), dtype=y.dtype, device=y.device)
+        attn_ops.paged_attention(qkv, heads, kv, batch, self.num_heads, self.num_kv_heads, self.head_dim, self.scale,
+                                 self.window, keep_first=self.keep_first, value_dim=self.value_dim)
+        if not direct:
+            if self.gate is None:
+                out[:, out_col0:out_col0 + self.inner_width] = heads * mul
+            else:
+                K.head_norm_gate(heads, None, 0.0, y, col0 + self.qkv_width, out, out_col0, self.num_heads,
+                                 self.value_dim, self.gate, mul)

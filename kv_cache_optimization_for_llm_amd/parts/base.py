@@ -264,6 +264,66 @@ class Mixer(Part):
         raise NotImplementedError
 
 
+class PendingSum(tuple):
+    """Branch outputs not yet added to the residual stream that enter it times a constant:
+    ``stream += scale * (sum of the outputs)``.  A plain tuple of outputs means ``scale`` 1."""
+
+    scale: float = 1.0
+
+    def __new__(cls, outputs, scale: float = 1.0):
+        self = super().__new__(cls, outputs)
+        self.scale = float(scale)
+        return self
+
+
+class ProjectedMixer(Mixer):
+    """A mixer of the form ``y = W_in x`` (one joined input projection) -> something per token and
+    head over ``y`` -> ``W_out inner``.  Written this way a mixer runs alone (:meth:`forward`) or side
+    by side with others on the same input (``parts.composite.SideBySide``), which then joins all
+    input projections into one product and all output projections into another: the mixer only
+    says what its input rows are, what it does between the two products, and where its state lies.
+
+    Subclasses set ``self.hidden_size`` and ``self.inner_width`` and implement
+    :meth:`input_weight`, :meth:`output_weight` (after ``load``) and :meth:`forward_inner`."""
+
+    hidden_size: int = 0
+    inner_width: int = 0
+
+    def input_weight(self) -> torch.Tensor:
+        """``[input columns, hidden]``: every matrix that reads the mixer's input, joined by rows."""
+        raise NotImplementedError
+
+    def output_weight(self) -> torch.Tensor:
+        """``[hidden, inner_width]``."""
+        raise NotImplementedError
+
+    def state_elements(self) -> int:
+        """fp32 values of state the mixer keeps per request (0: none)."""
+        return 0
+
+    def forward_inner(self, y: torch.Tensor, col0: int, ctx: MixerContext, state_off: int, out: torch.Tensor,
+                      out_col0: int, mul: float) -> None:
+        """``y`` ``[T, >= col0 + input columns]`` holds this mixer's projection from column ``col0`` on;
+        writes ``mul`` times what the output projection reads into columns ``out_col0 ..`` of ``out``.
+        The mixer's state lies at ``state_off`` of every row of ``ctx.state`` ``[seats, n]``."""
+        raise NotImplementedError
+
+    def state_spec(self) -> Optional[StateSpec]:
+        n = self.state_elements()
+        return StateSpec((n,), torch.float32) if n else None
+
+    def load_projections(self) -> None:
+        """Called at the end of a subclass's ``load``: the two products of the mixer run alone."""
+        from .linear import Linear
+        self._in, self._out = Linear(self.input_weight()), Linear(self.output_weight())
+
+    def forward(self, x: torch.Tensor, ctx: MixerContext) -> torch.Tensor:
+        y = self._in(x)
+        inner = torch.empty((x.shape[0], self.inner_width), dtype=x.dtype, device=x.device)
+        self.forward_inner(y, 0, ctx, 0, inner, 0, 1.0)
+        return self._out(inner)
+
+
 class FeedForward(Part):
     fuses_tail = False
 

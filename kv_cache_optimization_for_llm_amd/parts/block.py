@@ -12,7 +12,7 @@ from typing import Optional
 import torch
 
 from ..config.registry import BLOCKS
-from .base import Block, BranchTail, MixerContext, Norm, NormedRows
+from .base import Block, BranchTail, MixerContext, Norm, NormedRows, PendingSum
 
 
 @BLOCKS.register("pre_norm")
@@ -57,14 +57,19 @@ class ParallelBlock(Block):
     between layers - in one pass over the stream, in the stream's own type (an fp32 stream stays
     fp32 whatever the branches compute in).  When both norms are of one form with the same width
     and eps (``forward_pair``), one pass writes both normalised copies.  A layer without a
-    feed-forward (``"none"``) names only the ``"mixer"`` norm."""
+    feed-forward (``"none"``) names only the ``"mixer"`` norm.
+
+    ``shared_norm``: the layer has one norm (``"mixer"``) and both branches read its output.
+    ``residual_mult`` m: the branches enter the stream as ``h += m (mixer + ffn)`` - the sum is
+    handed on as a :class:`PendingSum` and the reader of the stream multiplies while it adds."""
 
     graph_safe = True
     NORM_NAMES = ("mixer", "feed_forward")
 
-    def __init__(self, mixer, feed_forward, norms):
+    def __init__(self, mixer, feed_forward, norms, *, shared_norm: bool = False, residual_mult: float = 1.0):
         self.has_ffn = not getattr(feed_forward, "absent", False)
-        if not self.has_ffn:
+        self.shared_norm, self.residual_mult = bool(shared_norm), float(residual_mult)
+        if not self.has_ffn or self.shared_norm:
             self.NORM_NAMES = ("mixer",)
         super().__init__(mixer, feed_forward, norms)
         self.mixer_norm = self.norms["mixer"]
@@ -77,13 +82,16 @@ class ParallelBlock(Block):
         if isinstance(delta, NormedRows):
             raise TypeError("a parallel block takes the stream and plain branch outputs, not prepared rows")
         pair = getattr(self.mixer_norm, "forward_pair", None)
-        if self.has_ffn and pair is not None and type(self.ffn_norm) is type(self.mixer_norm) \
+        if self.shared_norm or not self.has_ffn:
+            xm = xf = self.mixer_norm.forward(hidden, delta=delta)
+        elif pair is not None and type(self.ffn_norm) is type(self.mixer_norm) \
                 and (self.ffn_norm.width, self.ffn_norm.eps) == (self.mixer_norm.width, self.mixer_norm.eps):
             xm, xf = pair(self.ffn_norm, hidden, delta=delta)
         else:
             xm = self.mixer_norm.forward(hidden, delta=delta)        # adds the pending outputs to the stream
-            xf = self.ffn_norm.forward(hidden) if self.has_ffn else None
+            xf = self.ffn_norm.forward(hidden)
         a = self.mixer.forward(xm, ctx)
-        if not self.has_ffn:
-            return hidden, a
-        return hidden, (a, self.feed_forward.forward(xf, ctx))
+        out = (a, self.feed_forward.forward(xf, ctx)) if self.has_ffn else (a,)
+        if self.residual_mult != 1.0:
+            return hidden, PendingSum(out, self.residual_mult)
+        return hidden, out if self.has_ffn else a

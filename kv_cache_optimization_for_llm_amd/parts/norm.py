@@ -59,18 +59,26 @@ class LayerNorm(Norm):
     graph_safe = True
 
     def __init__(self, prefix: str, *, width: int, eps: float, weight_name: str = "weight",
-                 out_dtype: Optional[str] = None):
+                 out_dtype: Optional[str] = None, center: bool = True, weight_offset: float = 0.0):
+        """``center=False``: the mean is not taken off (``x / sqrt(mean(x^2) + eps) * w``, an RMS norm
+        over a stream of another type than the products').  ``weight_offset``: the weight is stored
+        around zero and multiplies as ``weight_offset + w`` (the sum is formed once, in 32-bit)."""
         super().__init__(prefix)
         self.width, self.eps = int(width), float(eps)
         self.weight_name = prefix + weight_name
         self.out_dtype = {None: None, "bfloat16": torch.bfloat16, "float32": torch.float32}[out_dtype]
+        self.center, self.weight_offset = bool(center), float(weight_offset)
         self.weight: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
-        return {self.weight_name: TensorSpec((self.width,), init="norm", role="vector")}
+        return {self.weight_name: TensorSpec((self.width,), init="zeros" if self.weight_offset else "norm", role="vector")}
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.weight = tensors[self.weight_name].contiguous()
+        if self.weight_offset:
+            if self.out_dtype is None:
+                self.out_dtype = self.weight.dtype          # the products behind the norm take the stored type
+            self.weight = (self.weight.float() + self.weight_offset).contiguous()
 
     def activation_elements(self) -> int:
         return self.width
@@ -81,6 +89,10 @@ class LayerNorm(Norm):
             return ()
         return tuple(delta) if isinstance(delta, (tuple, list)) else (delta,)
 
+    @staticmethod
+    def _scale(delta) -> float:
+        return float(getattr(delta, "scale", 1.0))
+
     def _out(self, x, row_idx):
         rows = x.shape[0] if row_idx is None else row_idx.shape[0]
         # the products behind a norm take the weights' type; a 32-bit stream of a bf16 model is normalised into bf16
@@ -88,11 +100,14 @@ class LayerNorm(Norm):
 
     def forward(self, x, out=None, delta=None, row_idx=None):
         out = self._out(x, row_idx) if out is None else out
-        return K.layernorm(x, self.weight, self.eps, out, deltas=self._deltas(delta), row_idx=row_idx)
+        return K.layernorm(x, self.weight, self.eps, out, deltas=self._deltas(delta), row_idx=row_idx,
+                           rms=not self.center, delta_scale=self._scale(delta))
 
     def forward_pair(self, twin: "LayerNorm", x, delta=None):
-        if twin.width != self.width or twin.eps != self.eps or twin.weight.dtype != self.weight.dtype:
-            raise ValueError("two norms share a pass only with the same width, eps and weight type")
+        if twin.width != self.width or twin.eps != self.eps or twin.weight.dtype != self.weight.dtype \
+                or twin.center != self.center:
+            raise ValueError("two norms share a pass only with the same form, width, eps and weight type")
         out, out2 = self._out(x, None), self._out(x, None)
-        K.layernorm(x, self.weight, self.eps, out, deltas=self._deltas(delta), weight2=twin.weight, out2=out2)
+        K.layernorm(x, self.weight, self.eps, out, deltas=self._deltas(delta), weight2=twin.weight, out2=out2,
+                    rms=not self.center, delta_scale=self._scale(delta))
         return out, out2

@@ -1,0 +1,184 @@
+"""Mixers that carry a state of fixed size per request instead of keys and values.
+
+Both are :class:`~.base.ProjectedMixer`: one joined input projection, a recurrence over the
+request's tokens in order (``csrc/recurrent.hip``: the state ``S [key channels, value channels]``
+of every head is fp32, lives in the seat's state row between steps, and everything that enters
+the recurrence - decays, step sizes, unit norms - is formed in fp32 from the projection), a norm
+of every head's read-out, a gate, and the output projection.  A prompt may be cut anywhere: the
+order of every sum depends on the sizes alone.
+
+* :class:`GatedLinearAttention` (``"gated_linear_attention"``):
+  ``S_t = diag(alpha_t) S_(t-1) + k_t v_t^T``, ``o_t = S_t^T q_t`` with a decay per key channel
+  ``alpha = sigmoid(z)^(1 / tau)``, ``z`` a low-rank projection of the input with a bias.
+* :class:`GatedDeltaRule` (``"gated_delta_rule"``): ``S <- g S; u = beta (v - S^T k); S <- S + k u^T;
+  o = S^T q`` with one decay ``g = exp(-exp(A_log) softplus(a + dt_bias))`` and one step size
+  ``beta = sigmoid(b)`` per head, unit-norm q and k, and a short causal convolution with silu on
+  q, k and v whose last inputs are part of the state.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from ..config.registry import MIXERS
+from ..models.spec import TensorSpec
+from ..ops import kernels as K
+from .base import MixerContext, ProjectedMixer
+from .linear import Linear
+
+
+def _names(defaults: Dict[str, str], given: Optional[Dict[str, str]], prefix: str) -> Dict[str, str]:
+    names = dict(defaults)
+    names.update(given or {})
+    return {key: prefix + name for key, name in names.items()}
+
+
+@MIXERS.register("gated_linear_attention")
+class GatedLinearAttention(ProjectedMixer):
+    graph_safe = True
+
+    def __init__(self, prefix: str, *, hidden_size: int, num_heads: int, head_dim: int, value_dim: int, tau: float,
+                 norm_eps: float, decay_rank: Optional[int] = None, query_scale: Optional[float] = None,
+                 tensor_names: Optional[Dict[str, str]] = None):
+        """``decay_rank``: the inner size of the decay's low-rank projection; ``None`` takes it from the
+        stored tensors.  ``query_scale``: what q is multiplied by (default ``head_dim^-1/2``).
+        ``tensor_names`` maps ``q k v g o norm a1 a2 a2_bias`` to names behind ``prefix``."""
+        super().__init__(prefix)
+        if tau <= 0:
+            raise ValueError(f"{prefix}: tau {tau} must be positive")
+        self.hidden_size, self.num_heads, self.head_dim, self.value_dim = int(hidden_size), int(num_heads), int(head_dim), int(value_dim)
+        self.tau, self.norm_eps = float(tau), float(norm_eps)
+        self.decay_rank = None if decay_rank is None else int(decay_rank)
+        self.query_scale = float(head_dim) ** -0.5 if query_scale is None else float(query_scale)
+        self.inner_width = self.num_heads * self.value_dim
+        self.names = _names(dict(q="q", k="k", v="v", g="g", o="o", norm="norm", a1="a1", a2="a2", a2_bias="a2.b"),
+                            tensor_names, prefix)
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        n, W, hd, hv, r = self.names, self.hidden_size, self.num_heads * self.head_dim, self.inner_width, self.decay_rank
+        return {
+            n["q"]: TensorSpec((hd, W)), n["k"]: TensorSpec((hd, W)), n["v"]: TensorSpec((hv, W)),
+            n["g"]: TensorSpec((hv, W)), n["o"]: TensorSpec((W, hv)),
+            n["norm"]: TensorSpec((self.value_dim,), init="norm", role="vector"),
+            n["a1"]: TensorSpec((r, W)), n["a2"]: TensorSpec((hd, r)),
+            n["a2_bias"]: TensorSpec((hd,), init="zeros", role="vector"),
+        }
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        t = {key: tensors[name] for key, name in self.names.items()}
+        if t["a1"].shape[0] != t["a2"].shape[1]:
+            raise ValueError(f"{self.prefix}: the decay's two matrices do not fit each other: "
+                             f"{tuple(t['a1'].shape)} and {tuple(t['a2'].shape)}")
+        self._w_in = torch.cat([t["q"], t["k"], t["v"], t["g"], t["a1"]], dim=0).contiguous()
+        self._w_out = t["o"]
+        self.rank = int(t["a1"].shape[0])
+        hd, hv = self.num_heads * self.head_dim, self.inner_width
+        self.q_off, self.k_off, self.v_off, self.g_off, self.a_off = 0, hd, 2 * hd, 2 * hd + hv, 2 * hd + 2 * hv
+        # decays are formed in 32-bit: the second matrix of the low-rank projection multiplies in fp32
+        self.a2 = Linear(t["a2"].float())
+        self.a2_bias = t["a2_bias"].float().contiguous()
+        self.norm_weight = t["norm"].float().contiguous()
+        self.load_projections()
+
+    def input_weight(self) -> torch.Tensor:
+        return self._w_in
+
+    def output_weight(self) -> torch.Tensor:
+        return self._w_out
+
+    def state_elements(self) -> int:
+        return self.num_heads * self.head_dim * self.value_dim
+
+    def activation_elements(self) -> int:
+        return 3 * self.num_heads * self.head_dim + 5 * self.inner_width + self.hidden_size
+
+    def forward_inner(self, y, col0, ctx: MixerContext, state_off, out, out_col0, mul) -> None:
+        batch, T = ctx.batch, y.shape[0]
+        low = y[:, col0 + self.a_off:col0 + self.a_off + self.rank].contiguous()
+        z = self.a2(low, out_dtype=torch.float32)
+        o = torch.empty((T, self.inner_width), dtype=torch.float32, device=y.device)
+        K.gated_linear_attention(y, col0 + self.q_off, col0 + self.k_off, col0 + self.v_off, z, self.a2_bias, self.tau,
+                                 self.query_scale, o, ctx.state, state_off, batch.entry_q_start, batch.entry_seat,
+                                 self.num_heads, self.head_dim, self.value_dim)
+        K.head_norm_gate(o, self.norm_weight, self.norm_eps, y, col0 + self.g_off, out, out_col0, self.num_heads,
+                         self.value_dim, "silu", mul)
+
+
+@MIXERS.register("gated_delta_rule")
+class GatedDeltaRule(ProjectedMixer):
+    graph_safe = True
+
+    def __init__(self, prefix: str, *, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 value_dim: int, conv_taps: int, norm_eps: float, unit_eps: float = 1e-6,
+                 tensor_names: Optional[Dict[str, str]] = None):
+        """``num_kv_heads`` query/key heads serve ``num_heads`` value heads (head h uses q/k head
+        ``h // (num_heads / num_kv_heads)``).  ``conv_taps``: length of the causal convolution on q, k, v
+        (1: none but the silu).  ``tensor_names`` maps ``q k v q_conv k_conv v_conv beta decay A_log dt_bias
+        g norm o`` to names behind ``prefix``."""
+        super().__init__(prefix)
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{prefix}: {num_heads} heads is not a multiple of {num_kv_heads} key heads")
+        if not 1 <= conv_taps <= 17:
+            raise ValueError(f"{prefix}: a convolution of {conv_taps} taps (1..17 are built)")
+        self.hidden_size, self.num_heads, self.num_kv_heads = int(hidden_size), int(num_heads), int(num_kv_heads)
+        self.head_dim, self.value_dim, self.conv_taps = int(head_dim), int(value_dim), int(conv_taps)
+        self.norm_eps, self.unit_eps = float(norm_eps), float(unit_eps)
+        self.inner_width = self.num_heads * self.value_dim
+        self.conv_channels = 2 * self.num_kv_heads * self.head_dim + self.inner_width
+        self.names = _names(dict(q="q", k="k", v="v", q_conv="q.conv", k_conv="k.conv", v_conv="v.conv", beta="b",
+                                 decay="a", A_log="A_log", dt_bias="dt_bias", g="g", norm="norm", o="o"),
+                            tensor_names, prefix)
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        n, W, gd, hv, H, taps = self.names, self.hidden_size, self.num_kv_heads * self.head_dim, self.inner_width, \
+            self.num_heads, self.conv_taps
+        return {
+            n["q"]: TensorSpec((gd, W)), n["k"]: TensorSpec((gd, W)), n["v"]: TensorSpec((hv, W)),
+            n["q_conv"]: TensorSpec((gd, taps), init="norm", role="vector"),
+            n["k_conv"]: TensorSpec((gd, taps), init="norm", role="vector"),
+            n["v_conv"]: TensorSpec((hv, taps), init="norm", role="vector"),
+            n["beta"]: TensorSpec((H, W)), n["decay"]: TensorSpec((H, W)),
+            n["A_log"]: TensorSpec((H,), init="zeros", role="vector"),
+            n["dt_bias"]: TensorSpec((H,), init="zeros", role="vector"),
+            n["g"]: TensorSpec((hv, W)), n["norm"]: TensorSpec((self.value_dim,), init="norm", role="vector"),
+            n["o"]: TensorSpec((W, hv)),
+        }
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        t = {key: tensors[name] for key, name in self.names.items()}
+        self._w_in = torch.cat([t["q"], t["k"], t["v"], t["beta"], t["decay"], t["g"]], dim=0).contiguous()
+        self._w_out = t["o"]
+        self.beta_off = self.conv_channels
+        self.decay_off = self.beta_off + self.num_heads
+        self.g_off = self.decay_off + self.num_heads
+        self.conv_weight = torch.cat([t["q_conv"], t["k_conv"], t["v_conv"]], dim=0).float().contiguous()
+        self.a_log, self.dt_bias = t["A_log"].float().contiguous(), t["dt_bias"].float().contiguous()
+        self.norm_weight = t["norm"].float().contiguous()
+        self.load_projections()
+
+    def input_weight(self) -> torch.Tensor:
+        return self._w_in
+
+    def output_weight(self) -> torch.Tensor:
+        return self._w_out
+
+    def state_elements(self) -> int:
+        # S of every head, then the convolution's last inputs
+        return self.num_heads * self.head_dim * self.value_dim + self.conv_channels * (self.conv_taps - 1)
+
+    def activation_elements(self) -> int:
+        return 3 * self.conv_channels + 4 * self.inner_width + self.hidden_size
+
+    def forward_inner(self, y, col0, ctx: MixerContext, state_off, out, out_col0, mul) -> None:
+        batch, T = ctx.batch, y.shape[0]
+        s_elems = self.num_heads * self.head_dim * self.value_dim
+        qkv = torch.empty((T, self.conv_channels), dtype=torch.float32, device=y.device)
+        K.causal_conv_act(y, col0, self.conv_weight, qkv, ctx.state, state_off + s_elems, batch.entry_q_start,
+                          batch.entry_seat, batch.max_q_len)
+        o = torch.empty((T, self.inner_width), dtype=torch.float32, device=y.device)
+        K.gated_delta_rule(qkv, y, col0 + self.beta_off, col0 + self.decay_off, self.a_log, self.dt_bias, o, ctx.state,
+                           state_off, batch.entry_q_start, batch.entry_seat, self.num_heads, self.num_kv_heads,
+                           self.head_dim, self.value_dim, self.unit_eps)
+        K.head_norm_gate(o, self.norm_weight, self.norm_eps, y, col0 + self.g_off, out, out_col0, self.num_heads,
+                         self.value_dim, "silu", mul)

@@ -94,7 +94,8 @@ def validate(index: Mapping[str, Tuple[str, dict]], specs: Mapping[str, TensorSp
             continue
         info = index[name][1]
         shape = tuple(info.get("shape", ()))
-        if shape != tuple(spec.shape):
+        # a size the model does not fix (None) is taken from the stored tensor
+        if len(shape) != len(spec.shape) or any(want is not None and want != got for want, got in zip(spec.shape, shape)):
             wrong_shape.append(f"{name}: stored {list(shape)}, the model needs {list(spec.shape)}")
         tag = info.get("dtype")
         ok = (tag in _INT_TAGS) if spec.role == "table" else (tag in _FLOAT_TAGS)
