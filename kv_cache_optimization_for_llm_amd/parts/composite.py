@@ -22,6 +22,8 @@ from .linear import Linear
 
 @MIXERS.register("side_by_side")
 class SideBySide(Mixer):
+    COLUMN_ALIGN = 8        # kernels that read a child's columns with wide loads need its rows aligned
+
     def __init__(self, prefix: str = "", *, hidden_size: int, children: Sequence[PartSpec], scales: Sequence[float]):
         super().__init__(prefix)
         self.hidden_size = int(hidden_size)
@@ -58,7 +60,11 @@ class SideBySide(Mixer):
         ins, outs = [], []
         for c in self.children:
             c.load(tensors)
-            ins.append(c.input_weight())
+            w = c.input_weight()
+            pad = -w.shape[0] % self.COLUMN_ALIGN
+            if pad:         # every child's columns start at a multiple of 16 (or 32) bytes of a row
+                w = torch.cat([w, w.new_zeros((pad, w.shape[1]))], dim=0)
+            ins.append(w)
             outs.append(c.output_weight())
         if len({w.dtype for w in ins + outs}) != 1:
             raise ValueError(f"{self.prefix}: the children's projection weights are stored in different dtypes")

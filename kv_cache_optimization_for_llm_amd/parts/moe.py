@@ -29,6 +29,9 @@ from .linear import Linear
 @FEED_FORWARDS.register("routed_experts")
 class RoutedExperts(FeedForward):
     graph_safe = True
+    # a function ``(part, idx [T, top] on the device)`` called after every routing of an eager step:
+    # for whoever wants to see which experts the tokens were sent to (tests do); None: nothing is called
+    on_route = None
 
     def __init__(self, prefix: str, *, hidden_size: int, intermediate_size: int, experts: int, top: int,
                  identity: int = 0, activation: str = "gelu", correction: bool = True, renormalise: bool = False,
@@ -77,6 +80,8 @@ class RoutedExperts(FeedForward):
         idx = torch.empty((T, self.top), dtype=torch.int32, device=dev)
         wgt = torch.empty((T, self.top), dtype=torch.float32, device=dev)
         K.moe_route(logits, self.correction, self.top, idx, wgt, self.renormalise)
+        if RoutedExperts.on_route is not None and not torch.cuda.is_current_stream_capturing():
+            RoutedExperts.on_route(self, idx)
         slots = T * self.top
         rows = torch.empty((slots, self.hidden_size), dtype=torch.float32, device=dev)
         if self.experts:

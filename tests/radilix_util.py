@@ -1,0 +1,210 @@
+"""Small Radilix configurations with seeded weights, and helpers that step an engine through a
+schedule and compare with the plain implementation (``plain_radilix``)."""
+import json
+import os
+from typing import Dict, List, Optional, Tuple
+
+import numpy as np
+import torch
+
+import plain_radilix as plain
+
+
+def moe(experts, top, ff, identity=0):
+    return {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "identity": identity, "top": top}}
+
+
+def gla_layer(heads, dim, vdim, tau, rank, mlp=None, **more):
+    return {"type": "gla", "mixer": {"heads": heads, "dim": dim, "vdim": vdim, "tau": tau, "decay_rank": rank},
+            "mlp": mlp, **more}
+
+
+def parallel_layer(left, right, left_scale, right_scale, mlp=None, **more):
+    h, g, d, dv, rot, base, scale = left
+    rh, rg, rd, rdv, conv = right
+    return {"type": "parallel", "mixer": {
+        "left": {"heads": h, "kv_heads": g, "dim": d, "vdim": dv, "rot": {"dims": rot, "base": base}, "scale": scale},
+        "right": {"heads": rh, "kv_heads": rg, "dim": rd, "vdim": rdv, "conv": conv},
+        "left_scale": left_scale, "right_scale": right_scale}, "mlp": mlp, **more}
+
+
+# The layers' eps is large in these configurations on purpose.  A head's read-out is divided by its own
+# root mean square; at a request's first token it is one value vector times q . k, and with a small eps
+# the sign of a q . k near zero decides a whole head: rounding to bfloat16 then moves a row by any
+# amount.  With eps of the order of the read-out itself the division is smooth there, every row is
+# well-conditioned in both formats, and an eps in the wrong place shows all the more.
+def shared(layer: dict, j: int) -> dict:
+    return {**layer, "weights_of": j}
+
+
+# A: values smaller than keys, a rotation over half of a head, three taps, a value size of the delta
+#    rule that is no multiple of 16; a gla layer without feed-forward; layer 2 runs with layer 0's weights;
+#    a router whose every output is chosen (top = experts, no identity experts).
+_A0 = parallel_layer((4, 2, 32, 16, 16, 10000.0, 0.2), (4, 2, 16, 24, 3), 0.8, 1.3, moe(5, 2, 48, identity=1))
+CFG_A = {"architecture": "Radilix", "vocab": 211, "width": 96, "norm": {"eps": 0.05}, "residual_mult": 0.6, "layers": [
+    _A0, gla_layer(3, 16, 8, 4.0, 6), shared(_A0, 0), gla_layer(2, 24, 40, 8.0, 5, moe(3, 3, 40))]}
+# B: a width that is no multiple of 32 (the experts' plain product kernel), residual_mult and both
+#    scales 1, as many kv heads as heads on both sides, a rotation over the whole head, no convolution
+#    (one tap), more identity experts than real ones and one choice per token; gla first and last.
+_B0 = gla_layer(5, 8, 12, 2.0, 3, moe(2, 1, 24, identity=3))
+CFG_B = {"architecture": "Radilix", "vocab": 157, "width": 72, "norm": {"eps": 0.1}, "residual_mult": 1.0, "layers": [
+    _B0, parallel_layer((3, 3, 20, 20, 20, 1000.0, 0.3), (2, 2, 8, 8, 1), 1.0, 1.0, moe(4, 2, 16)),
+    parallel_layer((2, 1, 16, 32, 8, 500.0, 0.25), (6, 3, 12, 20, 5), 0.5, 2.0), shared(_B0, 0)]}
+# C: sizes at which the bf16 engine takes its matrix-core kernels: heads of 64 with 4 query heads a kv
+#    head, values of 32 beside keys of 64, experts of width 128 over a width of 256; two layers share
+#    weights with an earlier one.
+_C0 = parallel_layer((8, 2, 64, 64, 32, 100000.0, 0.125), (4, 2, 64, 64, 4), 1.1, 0.7, moe(8, 3, 128, identity=2))
+_C1 = gla_layer(4, 64, 64, 16.0, 16, moe(6, 2, 96, identity=1))
+CFG_C = {"architecture": "Radilix", "vocab": 257, "width": 256, "norm": {"eps": 0.02}, "residual_mult": 0.7, "layers": [
+    _C0, _C1, parallel_layer((4, 4, 64, 32, 64, 7000.0, 0.11), (2, 1, 32, 128, 2), 0.9, 0.9, moe(4, 1, 64, identity=1)),
+    shared(_C1, 1), shared(_C0, 0)]}
+CONFIGS = {"A": (CFG_A, 5), "B": (CFG_B, 6), "C": (CFG_C, 7)}
+
+
+def write_model(folder: str, cfg: dict, seed: int, gain: float = 1.0, edit=None) -> Tuple[str, Dict[str, torch.Tensor]]:
+    """A model folder with seeded weights: matrices N(0, gain / sqrt(in)); what the random-weights mode
+    leaves at zero or near one is spread out here so that it weighs in (norm weights around zero,
+    biases, convolution taps, decay rates, the routers' corrections).  ``edit(state)`` may change the
+    tensors before they are stored.  Returns the folder and the tensors as stored."""
+    from safetensors.torch import save_file
+    from kv_cache_optimization_for_llm_amd.models.builder import tensor_specs_for_config
+    from kv_cache_optimization_for_llm_amd.weights.random_init import random_state_dict
+
+    os.makedirs(folder, exist_ok=True)
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    state = random_state_dict(tensor_specs_for_config(cfg), seed, torch.bfloat16, gain)
+    g = torch.Generator().manual_seed(seed)
+
+    def rnd(shape, std, mean=0.0):
+        return (torch.randn(shape, generator=g) * std + mean).to(torch.bfloat16)
+    for name, t in state.items():
+        if name.endswith("norm1") or name == "final.norm":
+            state[name] = rnd(t.shape, 0.3)
+        elif name.endswith((".q.b", ".k.b", ".v.b")):
+            state[name] = rnd(t.shape, 0.5)
+        elif name.endswith(".conv"):
+            state[name] = rnd(t.shape, 0.6)
+        elif name.endswith(".A_log"):
+            state[name] = rnd(t.shape, 0.7, -1.0)
+        elif name.endswith(".dt_bias"):
+            state[name] = rnd(t.shape, 0.5)
+        elif name.endswith(".a2.b"):
+            state[name] = rnd(t.shape, 1.0, 2.0)
+        elif name.endswith(".correction"):
+            state[name] = rnd(t.shape, 0.1)
+    if edit is not None:
+        edit(state)
+    save_file(state, os.path.join(folder, "model.safetensors"))
+    return folder, state
+
+
+def prompt(cfg: dict, length: int, seed: int) -> List[int]:
+    return [int(t) for t in np.random.default_rng(seed).integers(0, cfg["vocab"], size=length)]
+
+
+def moe_calls(cfg: dict) -> List[int]:
+    """Indices of the layers (calls) that have a feed-forward, in run order."""
+    return [i for i, layer in enumerate(cfg["layers"]) if layer.get("mlp")]
+
+
+def run_steps(engine, steps: List[dict], cfg: Optional[dict] = None):
+    """Feeds trace steps (``replay_util``'s format) to ``engine.step`` and returns
+    {(request, position): logits row}; with ``cfg`` also {request: {layer: [T, top] chosen experts}}, as
+    the engine's routers chose (eager steps only)."""
+    from kv_cache_optimization_for_llm_amd.engine.batch import StepEntry
+    from kv_cache_optimization_for_llm_amd.parts.moe import RoutedExperts
+    pos: Dict[str, int] = {}
+    rows: Dict[Tuple[str, int], np.ndarray] = {}
+    routes: Dict[str, Dict[int, list]] = {}
+    calls = moe_calls(cfg) if cfg is not None else []
+    seen: list = []
+    if cfg is not None:
+        RoutedExperts.on_route = lambda part, idx: seen.append(idx.cpu().long())
+    try:
+        for st in steps:
+            del seen[:]
+            entries = [StepEntry(e["id"], e["tokens"], e.get("want", [])) for e in st["entries"]]
+            logits = engine.step(entries).float().cpu().numpy()
+            wanted = [(e["id"], pos.get(e["id"], 0) + i) for e in st["entries"] for i in e.get("want", [])]
+            assert logits.shape[0] == len(wanted)
+            for key, row in zip(wanted, logits):
+                rows[key] = row.copy()
+            if cfg is not None:
+                assert len(seen) == len(calls), "one routing per layer call with a feed-forward"
+                at = 0
+                for e in st["entries"]:
+                    n = len(e["tokens"])
+                    per = routes.setdefault(e["id"], {})
+                    for layer, idx in zip(calls, seen):
+                        per.setdefault(layer, []).append(idx[at:at + n])
+                    at += n
+            for e in st["entries"]:
+                pos[e["id"]] = pos.get(e["id"], 0) + len(e["tokens"])
+            for rid in st.get("end", []):
+                pos.pop(rid, None)
+                engine.release(rid)
+    finally:
+        RoutedExperts.on_route = None
+    if cfg is None:
+        return rows
+    return rows, {rid: {layer: torch.cat(parts) for layer, parts in per.items()} for rid, per in routes.items()}
+
+
+def row_error(got: np.ndarray, want: np.ndarray) -> float:
+    """Root mean square of the difference with its mean taken off, relative to the spread of the
+    expected row."""
+    d = got.astype(np.float64) - want.astype(np.float64)
+    d -= d.mean()
+    w = want.astype(np.float64) - want.mean()
+    return float(np.sqrt((d ** 2).mean()) / max(np.sqrt((w ** 2).mean()), 1e-12))
+
+
+TOLERANCE = {"float32": 2e-4, "bfloat16": 6e-2}
+LIMITS: Dict[str, List[float]] = {}      # per request and position, where expected_rows found a row ill-conditioned
+# a router's choice is the engine's to make where the plain implementation's own margin is below
+# this (the engine's input to the router carries its format's rounding)
+CLOSE_CALL = {"float32": 1e-4, "bfloat16": 5e-2}
+
+
+def expected_rows(cfg: dict, state: Dict[str, torch.Tensor], requests: Dict[str, List[int]], routes=None,
+                  dtype: str = "float32") -> Dict[str, np.ndarray]:
+    """Logits of the plain forward pass per request.  With ``routes`` (what the engine's routers chose)
+    the plain experts are the engine's, and every choice that differs from the plain router's own
+    must be a close call of that router."""
+    W = plain.to_f64(state)
+    out = {}
+    LIMITS.clear()
+    for rid, toks in requests.items():
+        forced = None
+        if routes is not None:
+            forced = {layer: idx[:len(toks)] for layer, idx in routes[rid].items()}
+        margins: dict = {}
+        out[rid] = plain.forward(cfg, W, toks, forced=forced, margins=margins).numpy()
+        if dtype == "bfloat16":
+            # the limit of a row is three times what rounding the norms', the projections' and the branches'
+            # outputs to bfloat16 does to it in the plain model, where that is more than the general limit
+            moved = plain.forward(cfg, W, toks, forced=forced, rounded=lambda t: t.to(torch.bfloat16).to(plain.F)).numpy()
+            LIMITS[rid] = [max(TOLERANCE[dtype], 3.0 * row_error(moved[p], out[rid][p])) for p in range(len(toks))]
+        if forced is not None:
+            for layer, (own, margin) in margins.items():
+                differs = (forced[layer].sort(-1).values != own.sort(-1).values).any(-1)
+                assert (margin[differs] <= CLOSE_CALL[dtype]).all(), \
+                    f"request {rid}, layer {layer}: the engine's router chose other experts where the choice was clear"
+    return out
+
+
+def assert_rows(rows, expected: Dict[str, np.ndarray], dtype: str, what: str = "") -> float:
+    """Every row within its limit in 32-bit.  In bfloat16 a row's limit is an estimate (one sample of
+    what rounding does at that place), so: no row beyond twice its limit, at most one in fifty (or one) beyond it."""
+    worst, over = 0.0, 0
+    for (rid, p), row in rows.items():
+        assert np.isfinite(row).all(), f"{what}: request {rid} position {p} has a logit that is not finite"
+        e = row_error(row, expected[rid][p])
+        limit = LIMITS[rid][p] if dtype == "bfloat16" and rid in LIMITS else TOLERANCE[dtype]
+        hard = 2.0 * limit if dtype == "bfloat16" else limit
+        assert e <= hard, f"{what}: request {rid} position {p} is off by {e:.3g} (limit {hard:.3g})"
+        over += e > limit
+        worst = max(worst, e)
+    assert over <= max(1, len(rows) // 50), f"{what}: {over} of {len(rows)} rows are beyond their limits"
+    return worst
