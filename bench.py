@@ -15,7 +15,7 @@ tokens, each with its step time, bytes and fraction of the HBM peak, and the ser
 (``kclass_...``; ``--no-kernel-classes`` leaves them out) and, for the serving runs, pages reused,
 preemptions and fragmentation failures.
 
-    python bench.py --design gadopel [--layers 8]
+    python bench.py --design gadopel|radilix [--layers 8]
 
 is another measurement with a JSON line of its own (the default run above is untouched): prefill
 and decode throughput of a Gadopel model at layer sizes of a served model (random weights), beside
@@ -87,6 +87,23 @@ def gadopel_config(layers: int, vocab: int) -> dict:
             "layers": [latent if i % 2 == 0 else windowed for i in range(layers)], "max_positions": 8192}
 
 
+# --design radilix: layers of width 2,048.  Three in four are mixers side by side - attention with
+# 32 heads of 64 over 8 kv heads (rotation of half a head, biases, sigmoid gate) beside a gated delta
+# rule with 8 value heads of 128 over 4 query/key heads of 128 and four taps -, every fourth is gated
+# linear attention with 16 heads of 64 x 128; every layer has 16 routed experts of width 1,024 and 2
+# identity experts, 4 choices a token (67 M expert weights a layer against the Llama layer's 50 M of
+# feed-forward; a token uses a quarter of them).
+def radilix_config(layers: int, vocab: int) -> dict:
+    mlp = {"kind": "moe", "expert": {"ff": 1024}, "router": {"experts": 16, "identity": 2, "top": 4}}
+    side = {"type": "parallel", "mlp": mlp, "mixer": {
+        "left": {"heads": 32, "kv_heads": 8, "dim": 64, "vdim": 64, "scale": 0.125, "rot": {"base": 500000.0, "dims": 32}},
+        "right": {"heads": 8, "kv_heads": 4, "dim": 128, "vdim": 128, "conv": 4},
+        "left_scale": 1.0, "right_scale": 0.5}}
+    gla = {"type": "gla", "mlp": mlp, "mixer": {"heads": 16, "dim": 64, "vdim": 128, "tau": 16.0, "decay_rank": 16}}
+    return {"architecture": "Radilix", "vocab": vocab, "width": 2048, "norm": {"eps": 1e-6}, "residual_mult": 0.7,
+            "layers": [gla if i % 4 == 3 else side for i in range(layers)], "max_positions": 8192}
+
+
 def design_comparison(args) -> int:
     import torch
     from kv_cache_optimization_for_llm_amd.engine.batch import StepEntry
@@ -95,7 +112,8 @@ def design_comparison(args) -> int:
 
     layers, vocab = args.layers or 8, 32000
     llama = dict(CONFIG_1B, num_hidden_layers=layers, vocab_size=vocab, tie_word_embeddings=False)
-    configs = {"gadopel": gadopel_config(layers, vocab), "llama": llama}
+    design = args.design
+    configs = {design: {"gadopel": gadopel_config, "radilix": radilix_config}[design](layers, vocab), "llama": llama}
     shapes = [(8, 4096), (32, 2048)]            # (requests, context) of the decode runs
     gen = torch.Generator().manual_seed(0)
     out = {}
@@ -104,8 +122,10 @@ def design_comparison(args) -> int:
         engine = Engine(None, EngineOptions(dtype="bfloat16", page_size=PAGE, cache_tokens=pool, max_seqs=32,
                                             max_seq_len=8192, max_batch_tokens=8192, max_logit_rows=64),
                         config_dict=cfg, random_seed=0)
+        stacked = [w for b in engine.model.blocks for w in (getattr(b.feed_forward, "w_up", None),
+                                                            getattr(b.feed_forward, "w_down", None)) if w is not None]
         res = {"weight_gb": round(sum(t.numel() * t.element_size() for t in
-                                      [lin.weight for lin in engine.model.linears()]) / 1e9, 3),
+                                      [lin.weight for lin in engine.model.linears()] + stacked) / 1e9, 3),
                "cache_bytes_per_token": engine.cache.page_bytes() // PAGE}
 
         def timed_prefill(tokens):
@@ -166,10 +186,10 @@ def design_comparison(args) -> int:
         gc.collect()
         torch.cuda.empty_cache()
     b, c = shapes[0]
-    print(json.dumps({"metric": "gadopel_decode_tokens_per_second", "value": out["gadopel"][f"decode_b{b}_c{c}_tok_s"],
+    print(json.dumps({"metric": f"{design}_decode_tokens_per_second", "value": out[design][f"decode_b{b}_c{c}_tok_s"],
                       "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
                       "higher_is_better": True, "dtype": "bf16", "data": "synthetic (random weights, seeded token ids)",
-                      "config": {"design": "gadopel beside llama", "layers": layers, "width": 2048, "ff": 8192,
+                      "config": {"design": f"{design} beside llama", "layers": layers, "width": 2048, "ff": 8192,
                                  "vocab": vocab, "decode_shapes": shapes, "prefill_tokens": PREFILL_TOKENS},
                       "designs": out}))
     return 0
@@ -177,7 +197,7 @@ def design_comparison(args) -> int:
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--design", choices=["gadopel"], default=None,
+    ap.add_argument("--design", choices=["gadopel", "radilix"], default=None,
                     help="another measurement (its own JSON line): a model of this design at the layer sizes of a "
                          "served model beside a Llama model of equal size; the default run is left as it is")
     ap.add_argument("--gpus", type=int, default=1)

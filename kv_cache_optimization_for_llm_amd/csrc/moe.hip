@@ -202,17 +202,20 @@ moe_expert_rows_kernel(MoeRows a, void *__restrict__ out, int out_dtype, const T
     }
 }
 
-// matrix cores: a wavefront takes a tile of 16 rows and NT tiles of 16 outputs; out^T[n, t] =
-// W[e][n, :] . x[t, :]; operands straight from memory, 16 bytes a lane and product
+// matrix cores: a workgroup takes a tile of 16 rows and NT tiles of 16 outputs; out^T[n, t] =
+// W[e][n, :] . x[t, :]; operands straight from memory, 16 bytes a lane and product.  Its four
+// wavefronts take a quarter of K each (the same quarters whatever NT and the batch are) and the
+// first adds the four partial results up in a fixed order: with few tiles - decoded tokens - there are
+// four times as many wavefronts streaming the experts' matrices.
 template <int NT>
 __global__ void __launch_bounds__(256)
 moe_expert_rows_mfma_kernel(MoeRows a, void *__restrict__ out, int out_dtype, const bf16_t *__restrict__ x,
                             const bf16_t *__restrict__ w) {
+    __shared__ float red[3][NT][KVA_WAVE][4];
     const int tile = blockIdx.y, e = a.tile_expert[tile];
     if (e < 0) return;
     const int lane = threadIdx.x % KVA_WAVE, wave = threadIdx.x / KVA_WAVE, r = lane & 15, g = lane >> 4;
-    const int n_first = (blockIdx.x * (blockDim.x / KVA_WAVE) + wave) * 16 * NT;
-    if (n_first >= a.N) return;
+    const int n_first = blockIdx.x * 16 * NT;
     const int place = tile * MOE_TILE + r, slot = a.sorted_slot[place];
     const size_t src = a.mode == 0 ? (size_t)(slot < 0 ? 0 : slot / a.top) : (size_t)place;
     const bf16_t *xrow = x + src * a.K + 8 * g;
@@ -223,7 +226,11 @@ moe_expert_rows_mfma_kernel(MoeRows a, void *__restrict__ out, int out_dtype, co
     f32x4 acc[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) acc[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
-    for (int k0 = 0; k0 < a.K; k0 += 32) {
+    const int steps = a.K / 32, per = (steps + 3) / 4;
+    const int s0 = wave * per, s1 = min(steps, s0 + per);
+#pragma unroll 4
+    for (int s = s0; s < s1; ++s) {
+        const int k0 = 32 * s;
         Frag8 xf, wf[NT];
         xf.u4 = *reinterpret_cast<const uint4 *>(xrow + k0);
 #pragma unroll
@@ -231,14 +238,21 @@ moe_expert_rows_mfma_kernel(MoeRows a, void *__restrict__ out, int out_dtype, co
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[nt].v, xf.v, acc[nt], 0, 0, 0);
     }
-    if (slot < 0) return;
+    if (wave > 0)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) red[wave - 1][nt][lane][i] = acc[nt][i];
+    __syncthreads();
+    if (wave > 0 || slot < 0) return;
     // lane (row r, group g) holds outputs n0 + 4 g .. + 3 of its row
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int n = n_first + 16 * nt + 4 * g + i;
-            if (n < a.N) moe_store(a, out, out_dtype, place, slot, n, acc[nt][i]);
+            const float v = ((acc[nt][i] + red[0][nt][lane][i]) + red[1][nt][lane][i]) + red[2][nt][lane][i];
+            if (n < a.N) moe_store(a, out, out_dtype, place, slot, n, v);
         }
 }
 
@@ -254,9 +268,13 @@ extern "C" int kva_moe_expert_rows(void *out, int out_dtype, const void *x, cons
     if (max_tiles == 0) return KVA_OK;
     MoeRows a{sorted_slot, tile_expert, slot_weight, top, N, K, mode, act};
     if (dtype == KVA_BF16 && K % 32 == 0) {
-        const int per_block = 4 * 16 * 4;
-        hipLaunchKernelGGL(moe_expert_rows_mfma_kernel<4>, dim3((N + per_block - 1) / per_block, max_tiles), dim3(256), 0,
-                           stream, a, out, out_dtype, (const bf16_t *)x, (const bf16_t *)w);
+        // few tiles: 16 outputs a workgroup, so that enough of them stream the matrices; many: 64, which share x
+        if ((long long)max_tiles * ((N + 15) / 16) <= 8192)
+            hipLaunchKernelGGL(moe_expert_rows_mfma_kernel<1>, dim3((N + 15) / 16, max_tiles), dim3(256), 0, stream, a,
+                               out, out_dtype, (const bf16_t *)x, (const bf16_t *)w);
+        else
+            hipLaunchKernelGGL(moe_expert_rows_mfma_kernel<4>, dim3((N + 63) / 64, max_tiles), dim3(256), 0, stream, a,
+                               out, out_dtype, (const bf16_t *)x, (const bf16_t *)w);
     } else if (dtype == KVA_BF16) {
         hipLaunchKernelGGL(moe_expert_rows_kernel<bf16_t>, dim3((N + 63) / 64, max_tiles), dim3(256), 0, stream, a, out,
                            out_dtype, (const bf16_t *)x, (const bf16_t *)w);
@@ -294,5 +312,103 @@ extern "C" int kva_moe_combine(void *out, const void *x, int dtype, const float 
     hipLaunchKernelGGL(moe_combine_kernel, dim3(tokens), dim3(256), 0, stream, out, x, dtype, rows, idx, wgt, width, top,
                        experts);
     KVA_CHECK_LAUNCH("moe_combine");
+    return KVA_OK;
+}
+
+// ---- small products with 32-bit results -------------------------------------------------------
+// out[t, n] = sum_k x[t, k] * w[n, k] in fp32, for the small matrices whose results must not be rounded
+// to 16 bits (a router's logits; the second half of a low-rank projection that makes decays, which
+// may be finished here: bias, sigmoid, power).  x and
+// w may be bf16 or fp32; every product and sum is fp32.  A workgroup takes a token: its row of x goes
+// to LDS once; with a long K a wavefront takes an output and its lanes stride over K (sum by
+// wavefront reduction), with a short K a thread takes an output.  The order of every sum depends on
+// the sizes alone.
+#define SMALL_PRODUCT_MAX_K 8192
+
+__device__ inline float moe_ld(const void *p, int dtype, size_t i) {
+    return dtype == KVA_BF16 ? bf16_bits_to_float(reinterpret_cast<const uint16_t *>(p)[i])
+                             : reinterpret_cast<const float *>(p)[i];
+}
+
+// eight neighbouring elements from index i on (i a multiple of 8: 16 or 32 aligned bytes)
+__device__ inline void moe_ld8(const void *p, int dtype, size_t i, float (&f)[8]) {
+    if (dtype == KVA_BF16) {
+        const uint4 v = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p) + i);
+        const unsigned u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            f[2 * j] = __uint_as_float(u[j] << 16);
+            f[2 * j + 1] = __uint_as_float(u[j] & 0xffff0000u);
+        }
+    } else {
+        const float4 a = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(p) + i);
+        const float4 b = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(p) + i + 4);
+        f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+    }
+}
+
+// the result as it is, plus a bias, or - with decay_inv_tau > 0 - turned into a decay:
+// sigmoid(z)^(1 / tau) = exp(-softplus(-z) / tau) with z = the sum plus its bias
+__device__ inline float small_product_finish(float acc, const float *bias, int n, float decay_inv_tau) {
+    const float z = acc + (bias ? bias[n] : 0.f);
+    if (decay_inv_tau <= 0.f) return z;
+    const float softplus = fmaxf(-z, 0.f) + log1pf(expf(-fabsf(z)));
+    return expf(-softplus * decay_inv_tau);
+}
+
+__global__ void __launch_bounds__(256)
+small_product_f32_kernel(float *__restrict__ out, const void *__restrict__ x, int x_dtype, int x_stride,
+                         const void *__restrict__ w, int w_dtype, int N, int K, int per_block,
+                         const float *__restrict__ bias, float decay_inv_tau) {
+    extern __shared__ float xs[];
+    const size_t t = blockIdx.x;
+    const int n_lo = blockIdx.y * per_block, n_hi = min(N, n_lo + per_block);
+    for (int k = threadIdx.x; k < K; k += blockDim.x) xs[k] = moe_ld(x, x_dtype, t * x_stride + k);
+    __syncthreads();
+    const int K8 = (K % 8 == 0) ? K : 0;          // the part read eight elements at a time
+    if (K >= 128) {
+        const int lane = threadIdx.x % KVA_WAVE, wave = threadIdx.x / KVA_WAVE, waves = blockDim.x / KVA_WAVE;
+        for (int n = n_lo + wave; n < n_hi; n += waves) {
+            float acc = 0.f;
+            for (int k = 8 * lane; k < K8; k += 8 * KVA_WAVE) {
+                float f[8];
+                moe_ld8(w, w_dtype, (size_t)n * K + k, f);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc += xs[k + i] * f[i];
+            }
+            for (int k = K8 + lane; k < K; k += KVA_WAVE) acc += xs[k] * moe_ld(w, w_dtype, (size_t)n * K + k);
+            acc = wave_sum(acc);
+            if (lane == 0) out[t * N + n] = small_product_finish(acc, bias, n, decay_inv_tau);
+        }
+    } else {
+        for (int n = n_lo + threadIdx.x; n < n_hi; n += blockDim.x) {
+            float acc = 0.f;
+            for (int k = 0; k < K8; k += 8) {
+                float f[8];
+                moe_ld8(w, w_dtype, (size_t)n * K + k, f);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc += xs[k + i] * f[i];
+            }
+            for (int k = K8; k < K; ++k) acc += xs[k] * moe_ld(w, w_dtype, (size_t)n * K + k);
+            out[t * N + n] = small_product_finish(acc, bias, n, decay_inv_tau);
+        }
+    }
+}
+
+extern "C" int kva_small_product_f32(float *out, const void *x, int x_dtype, int x_stride, const void *w, int w_dtype,
+                                     int tokens, int N, int K, const float *bias, float decay_inv_tau,
+                                     hipStream_t stream) {
+    KVA_REQUIRE(out && x && w && tokens >= 0 && N > 0, "small_product_f32: missing operand or bad sizes");
+    KVA_REQUIRE(K > 0 && K <= SMALL_PRODUCT_MAX_K && x_stride >= K, "small_product_f32: K %d must lie in 1..%d", K, SMALL_PRODUCT_MAX_K);
+    KVA_REQUIRE((x_dtype == KVA_BF16 || x_dtype == KVA_F32) && (w_dtype == KVA_BF16 || w_dtype == KVA_F32),
+                "small_product_f32: unsupported dtype");
+    if (tokens == 0) return KVA_OK;
+    KVA_REQUIRE((reinterpret_cast<uintptr_t>(w) & 31) == 0, "small_product_f32: the matrix must be aligned to 32 bytes");
+    const int per_block = K >= 128 ? 16 : 256;         // outputs a workgroup: four a wavefront, or one a thread
+    const int blocks_y = (N + per_block - 1) / per_block;
+    KVA_REQUIRE(tokens <= 0x7fffffff && blocks_y <= 65535, "small_product_f32: too many outputs");
+    hipLaunchKernelGGL(small_product_f32_kernel, dim3(tokens, blocks_y), dim3(256), (size_t)K * sizeof(float), stream,
+                       out, x, x_dtype, x_stride, w, w_dtype, N, K, per_block, bias, decay_inv_tau);
+    KVA_CHECK_LAUNCH("small_product_f32");
     return KVA_OK;
 }

@@ -203,12 +203,11 @@ gated_delta_rule_kernel(RecArgs a, const float *__restrict__ qkv, int conv_strid
         for (int i = r; i < d; i += REC_ROWGROUPS) Sg[(size_t)i * dv + col] = S[i * REC_COLS + c];
 }
 
-// Gated linear attention.  q, k, v and the decay's input z are columns of y (heads x dim, heads x
-// dim, heads x vdim, heads x dim; z may live in another buffer); q is multiplied by q_mul.
+// Gated linear attention.  q, k, v are columns of y (heads x dim, heads x dim, heads x vdim); the
+// decays alpha (heads x dim a token, fp32) come in a buffer of their own; q is multiplied by q_mul.
 __global__ void __launch_bounds__(KVA_WAVE)
 gated_linear_attention_kernel(RecArgs a, const void *__restrict__ y, int y_dtype, int y_stride, int q_off, int k_off,
-                              int v_off, const void *__restrict__ z, int z_dtype, int z_stride, int z_off,
-                              const float *__restrict__ z_bias, float inv_tau, float q_mul) {
+                              int v_off, const float *__restrict__ alpha, int alpha_stride, float q_mul) {
     extern __shared__ float lds[];
     const int lane = threadIdx.x, c = lane % REC_COLS, r = lane / REC_COLS;
     const int slices = (a.vdim + REC_COLS - 1) / REC_COLS;
@@ -229,8 +228,7 @@ gated_linear_attention_kernel(RecArgs a, const void *__restrict__ y, int y_dtype
             const int i = head * d + x % d;
             qs[x] = rec_ld(y, y_dtype, row * y_stride + q_off + i) * q_mul;
             ks[x] = rec_ld(y, y_dtype, row * y_stride + k_off + i);
-            const float zz = rec_ld(z, z_dtype, row * z_stride + z_off + i) + z_bias[i];
-            as[x] = expf(-rec_softplus(-zz) * inv_tau);            // sigmoid(z)^(1 / tau)
+            as[x] = alpha[row * alpha_stride + i];
         }
         __syncthreads();
         for (int tt = 0; tt < m; ++tt) {
@@ -249,6 +247,227 @@ gated_linear_attention_kernel(RecArgs a, const void *__restrict__ y, int y_dtype
     }
     if (on)
         for (int i = r; i < d; i += REC_ROWGROUPS) Sg[(size_t)i * dv + col] = S[i * REC_COLS + c];
+}
+
+// ---- the two recurrences with the state in registers (key sizes up to 128) ----------------------
+// A wavefront takes 4 value columns of a head; the 16 lanes of a row of the wavefront share a
+// column.  Lane (c, r) owns, of column c, the rows 4 (16 j + r) .. + 3 for j < RP / 4 in RP
+// registers (rows from `dim` on are padding and stay zero): a 16-byte LDS read per j and lane takes
+// 256 neighbouring bytes of a token's k, q or alpha, and a sum over the rows ends with four
+// rotations inside the lanes' row.  A chunk of 16 tokens is staged in LDS - q, k (and the decays)
+// padded to 16 RP elements a token, the 4 values of the wavefront's columns, the token's two numbers;
+// the next chunk's global loads are issued before the current one is walked.  A head's columns are
+// spread over vdim / 4 wavefronts: a prompt of one request fills the chip at the sizes of a model.
+#define REC_CHUNK 16
+#define REG_COLS 4
+#define REG_LANES 16         // lanes that share a column
+
+template <int RP>
+__global__ void __launch_bounds__(KVA_WAVE)
+gated_delta_rule_reg_kernel(RecArgs a, const float *__restrict__ qkv, int conv_stride, const void *__restrict__ y,
+                            int y_dtype, int y_stride, int beta_off, int decay_off, const float *__restrict__ a_log,
+                            const float *__restrict__ dt_bias, float unit_eps) {
+    constexpr int DP = REG_LANES * RP, DS = DP + 4, CH = REC_CHUNK, PER = CH * DP / KVA_WAVE;   // token rows 4 banks apart
+    __shared__ __attribute__((aligned(16))) float qs[CH * DS];
+    __shared__ __attribute__((aligned(16))) float ks[CH * DS];
+    __shared__ float vs[CH * REG_COLS], bs[CH], gs[CH], nq[CH], nk[CH];
+    const int lane = threadIdx.x, c = lane / REG_LANES, r = lane % REG_LANES;
+    const int slices = (a.vdim + REG_COLS - 1) / REG_COLS;
+    const int head = blockIdx.x / slices, col0 = (blockIdx.x % slices) * REG_COLS, col = col0 + c;
+    const int e = blockIdx.y;
+    const int q0 = a.entry_q_start[e], n = a.entry_q_start[e + 1] - q0;
+    if (n <= 0) return;
+    const int d = a.dim, dv = a.vdim, kvh = head / (a.heads / a.kv_heads);
+    const bool on = col < dv;
+    float *Sg = a.state + (size_t)a.entry_seat[e] * a.seat_stride + a.state_off + (size_t)head * d * dv;
+    float S[RP];
+#pragma unroll
+    for (int j = 0; j < RP; ++j) {
+        const int i = 4 * (REG_LANES * (j / 4) + r) + j % 4;
+        S[j] = (on && i < d) ? Sg[(size_t)i * dv + col] : 0.f;
+    }
+    const int k_col = a.kv_heads * d, v_col = 2 * a.kv_heads * d;
+    const float rate = expf(a_log[head]), bias = dt_bias[head], q_mul = 1.0f / sqrtf((float)d);
+    float pq[PER], pk[PER], pv = 0.f, pb = 0.f, pg = 0.f;
+    auto fetch = [&](int t0, int m) {
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            pq[j] = pk[j] = 0.f;
+            if (KVA_WAVE * j / DP >= m) continue;           // (the whole wavefront: a decoded token loads one row)
+            const int x = lane + KVA_WAVE * j, tt = x / DP, i = x % DP;
+            if (i >= d) continue;
+            const size_t row = (size_t)(q0 + t0 + tt) * conv_stride;
+            pq[j] = qkv[row + kvh * d + i];
+            pk[j] = qkv[row + k_col + kvh * d + i];
+        }
+        {   // 16 tokens x 4 columns: one value a lane
+            const int tt = lane / REG_COLS, cc = lane % REG_COLS;
+            pv = (tt < m && col0 + cc < dv) ? qkv[(size_t)(q0 + t0 + tt) * conv_stride + v_col + head * dv + col0 + cc] : 0.f;
+        }
+        if (lane < m) {
+            const size_t yrow = (size_t)(q0 + t0 + lane) * y_stride;
+            pb = rec_ld(y, y_dtype, yrow + beta_off + head);
+            pg = rec_ld(y, y_dtype, yrow + decay_off + head);
+        }
+    };
+    fetch(0, min(CH, n));
+    for (int t0 = 0; t0 < n; t0 += CH) {
+        const int m = min(CH, n - t0);
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const int x = lane + KVA_WAVE * j, at = (x / DP) * DS + x % DP;
+            qs[at] = pq[j];
+            ks[at] = pk[j];
+        }
+        vs[lane] = pv;
+        if (lane < m) {
+            bs[lane] = rec_sigmoid(pb);
+            gs[lane] = expf(-rate * rec_softplus(pg + bias));
+        }
+        __syncthreads();
+        {   // what makes q and k unit vectors: token tt by the four lanes 4 tt .. 4 tt + 3, every fourth element each
+            const int tt = lane / 4, part = lane % 4;
+            float sq = 0.f, sk = 0.f;
+            if (tt < m)
+                for (int i = part; i < DP; i += 4) {
+                    sq += qs[tt * DS + i] * qs[tt * DS + i];
+                    sk += ks[tt * DS + i] * ks[tt * DS + i];
+                }
+            sq += __shfl_xor(sq, 1, KVA_WAVE); sq += __shfl_xor(sq, 2, KVA_WAVE);
+            sk += __shfl_xor(sk, 1, KVA_WAVE); sk += __shfl_xor(sk, 2, KVA_WAVE);
+            if (part == 0) {
+                nq[tt] = q_mul / sqrtf(sq + unit_eps);
+                nk[tt] = 1.0f / sqrtf(sk + unit_eps);
+            }
+        }
+        __syncthreads();
+        if (t0 + CH < n) fetch(t0 + CH, min(CH, n - t0 - CH));
+        for (int tt = 0; tt < m; ++tt) {
+            const float4 *k4 = reinterpret_cast<const float4 *>(ks + tt * DS) + r;
+            const float4 *q4 = reinterpret_cast<const float4 *>(qs + tt * DS) + r;
+            const float g = gs[tt], beta = bs[tt], v = vs[tt * REG_COLS + c], mq = nq[tt], mk = nk[tt];
+            // the unit vectors' factors multiply the sums: S^T (mk k) = mk (S^T k), S^T (mq q) likewise
+            float4 kk[RP / 4];
+            float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
+#pragma unroll
+            for (int j = 0; j < RP / 4; ++j) {
+                kk[j] = k4[REG_LANES * j];
+                kk[j].x *= mk; kk[j].y *= mk; kk[j].z *= mk; kk[j].w *= mk;
+                d0 += S[4 * j] * kk[j].x;
+                d1 += S[4 * j + 1] * kk[j].y;
+                d2 += S[4 * j + 2] * kk[j].z;
+                d3 += S[4 * j + 3] * kk[j].w;
+            }
+            const float dot = row16_sum((d0 + d1) + (d2 + d3));
+            const float u = beta * (v - g * dot);
+            float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
+#pragma unroll
+            for (int j = 0; j < RP / 4; ++j) {
+                const float4 qq = q4[REG_LANES * j];
+                S[4 * j] = g * S[4 * j] + kk[j].x * u;
+                S[4 * j + 1] = g * S[4 * j + 1] + kk[j].y * u;
+                S[4 * j + 2] = g * S[4 * j + 2] + kk[j].z * u;
+                S[4 * j + 3] = g * S[4 * j + 3] + kk[j].w * u;
+                o0 += S[4 * j] * qq.x;
+                o1 += S[4 * j + 1] * qq.y;
+                o2 += S[4 * j + 2] * qq.z;
+                o3 += S[4 * j + 3] * qq.w;
+            }
+            const float o = row16_sum((o0 + o1) + (o2 + o3)) * mq;
+            if (on && r == 0) a.out[(size_t)(q0 + t0 + tt) * a.heads * dv + head * dv + col] = o;
+        }
+    }
+    if (on)
+#pragma unroll
+        for (int j = 0; j < RP; ++j) {
+            const int i = 4 * (REG_LANES * (j / 4) + r) + j % 4;
+            if (i < d) Sg[(size_t)i * dv + col] = S[j];
+        }
+}
+
+template <int RP>
+__global__ void __launch_bounds__(KVA_WAVE)
+gated_linear_attention_reg_kernel(RecArgs a, const void *__restrict__ y, int y_dtype, int y_stride, int q_off, int k_off,
+                                  int v_off, const float *__restrict__ alpha, int alpha_stride, float q_mul) {
+    constexpr int DP = REG_LANES * RP, DS = DP + 4, CH = REC_CHUNK, PER = CH * DP / KVA_WAVE;   // token rows 4 banks apart
+    __shared__ __attribute__((aligned(16))) float qs[CH * DS];
+    __shared__ __attribute__((aligned(16))) float ks[CH * DS];
+    __shared__ __attribute__((aligned(16))) float as[CH * DS];
+    __shared__ float vs[CH * REG_COLS];
+    const int lane = threadIdx.x, c = lane / REG_LANES, r = lane % REG_LANES;
+    const int slices = (a.vdim + REG_COLS - 1) / REG_COLS;
+    const int head = blockIdx.x / slices, col0 = (blockIdx.x % slices) * REG_COLS, col = col0 + c;
+    const int e = blockIdx.y;
+    const int q0 = a.entry_q_start[e], n = a.entry_q_start[e + 1] - q0;
+    if (n <= 0) return;
+    const int d = a.dim, dv = a.vdim;
+    const bool on = col < dv;
+    float *Sg = a.state + (size_t)a.entry_seat[e] * a.seat_stride + a.state_off + (size_t)head * d * dv;
+    float S[RP];
+#pragma unroll
+    for (int j = 0; j < RP; ++j) {
+        const int i = 4 * (REG_LANES * (j / 4) + r) + j % 4;
+        S[j] = (on && i < d) ? Sg[(size_t)i * dv + col] : 0.f;
+    }
+    float pq[PER], pk[PER], pa[PER], pv = 0.f;
+    auto fetch = [&](int t0, int m) {
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            pq[j] = pk[j] = pa[j] = 0.f;
+            if (KVA_WAVE * j / DP >= m) continue;           // (the whole wavefront: a decoded token loads one row)
+            const int x = lane + KVA_WAVE * j, tt = x / DP, i = x % DP;
+            if (i >= d) continue;
+            const size_t row = (size_t)(q0 + t0 + tt);
+            pq[j] = rec_ld(y, y_dtype, row * y_stride + q_off + head * d + i);
+            pk[j] = rec_ld(y, y_dtype, row * y_stride + k_off + head * d + i);
+            pa[j] = alpha[row * alpha_stride + head * d + i];
+        }
+        const int tt = lane / REG_COLS, cc = lane % REG_COLS;
+        pv = (tt < m && col0 + cc < dv) ? rec_ld(y, y_dtype, (size_t)(q0 + t0 + tt) * y_stride + v_off + head * dv + col0 + cc) : 0.f;
+    };
+    fetch(0, min(CH, n));
+    for (int t0 = 0; t0 < n; t0 += CH) {
+        const int m = min(CH, n - t0);
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const int x = lane + KVA_WAVE * j, at = (x / DP) * DS + x % DP;
+            qs[at] = pq[j] * q_mul;
+            ks[at] = pk[j];
+            as[at] = pa[j];
+        }
+        vs[lane] = pv;
+        __syncthreads();
+        if (t0 + CH < n) fetch(t0 + CH, min(CH, n - t0 - CH));
+        for (int tt = 0; tt < m; ++tt) {
+            const float4 *k4 = reinterpret_cast<const float4 *>(ks + tt * DS) + r;
+            const float4 *q4 = reinterpret_cast<const float4 *>(qs + tt * DS) + r;
+            const float4 *a4 = reinterpret_cast<const float4 *>(as + tt * DS) + r;
+            const float v = vs[tt * REG_COLS + c];
+            float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
+#pragma unroll
+            for (int j = 0; j < RP / 4; ++j) {
+                const float4 kk = k4[REG_LANES * j], qq = q4[REG_LANES * j], al = a4[REG_LANES * j];
+                S[4 * j] = al.x * S[4 * j] + kk.x * v;
+                S[4 * j + 1] = al.y * S[4 * j + 1] + kk.y * v;
+                S[4 * j + 2] = al.z * S[4 * j + 2] + kk.z * v;
+                S[4 * j + 3] = al.w * S[4 * j + 3] + kk.w * v;
+                o0 += S[4 * j] * qq.x;
+                o1 += S[4 * j + 1] * qq.y;
+                o2 += S[4 * j + 2] * qq.z;
+                o3 += S[4 * j + 3] * qq.w;
+            }
+            const float o = row16_sum((o0 + o1) + (o2 + o3));
+            if (on && r == 0) a.out[(size_t)(q0 + t0 + tt) * a.heads * dv + head * dv + col] = o;
+        }
+    }
+    if (on)
+#pragma unroll
+        for (int j = 0; j < RP; ++j) {
+            const int i = 4 * (REG_LANES * (j / 4) + r) + j % 4;
+            if (i < d) Sg[(size_t)i * dv + col] = S[j];
+        }
 }
 
 static int rec_chunk(int dim, int arrays) {
@@ -276,6 +495,18 @@ extern "C" int kva_gated_delta_rule(float *out, float *state, long long seat_str
     if (int rc = rec_check("gated_delta_rule", out, state, entry_q_start, entry_seat, entries, heads, kv_heads, dim, vdim)) return rc;
     KVA_REQUIRE(qkv && y && a_log && dt_bias, "gated_delta_rule: missing operand");
     if (entries == 0) return KVA_OK;
+    if (dim <= 128) {
+        RecArgs a{out, state, (size_t)seat_stride, state_off, entry_q_start, entry_seat, heads, kv_heads, dim, vdim, REC_CHUNK};
+        const dim3 grid(heads * ((vdim + REG_COLS - 1) / REG_COLS), entries);
+#define KVA_DELTA_REG(RP)                                                                                              \
+    hipLaunchKernelGGL(gated_delta_rule_reg_kernel<RP>, grid, dim3(KVA_WAVE), 0, stream, a, qkv, conv_stride, y,       \
+                       y_dtype, y_stride, beta_off, decay_off, a_log, dt_bias, unit_eps)
+        if (dim <= 64) KVA_DELTA_REG(4);
+        else KVA_DELTA_REG(8);
+#undef KVA_DELTA_REG
+        KVA_CHECK_LAUNCH("gated_delta_rule");
+        return KVA_OK;
+    }
     const int chunk = rec_chunk(dim, 2);
     KVA_REQUIRE(chunk > 0, "gated_delta_rule: key size %d does not fit the LDS", dim);
     RecArgs a{out, state, (size_t)seat_stride, state_off, entry_q_start, entry_seat, heads, kv_heads, dim, vdim, chunk};
@@ -289,19 +520,31 @@ extern "C" int kva_gated_delta_rule(float *out, float *state, long long seat_str
 
 extern "C" int kva_gated_linear_attention(float *out, float *state, long long seat_stride, int state_off,
                                           const void *y, int y_dtype, int y_stride, int q_off, int k_off, int v_off,
-                                          const void *z, int z_dtype, int z_stride, int z_off, const float *z_bias,
-                                          float tau, float q_mul, const int *entry_q_start, const int *entry_seat,
+                                          const float *alpha, int alpha_stride, float q_mul,
+                                          const int *entry_q_start, const int *entry_seat,
                                           int entries, int heads, int dim, int vdim, hipStream_t stream) {
     if (int rc = rec_check("gated_linear_attention", out, state, entry_q_start, entry_seat, entries, heads, heads, dim, vdim)) return rc;
-    KVA_REQUIRE(y && z && z_bias && tau > 0.f, "gated_linear_attention: missing operand or tau <= 0");
+    KVA_REQUIRE(y && alpha && alpha_stride >= heads * dim, "gated_linear_attention: missing operand");
     if (entries == 0) return KVA_OK;
+    if (dim <= 128) {
+        RecArgs a{out, state, (size_t)seat_stride, state_off, entry_q_start, entry_seat, heads, heads, dim, vdim, REC_CHUNK};
+        const dim3 grid(heads * ((vdim + REG_COLS - 1) / REG_COLS), entries);
+#define KVA_GLA_REG(RP)                                                                                                \
+    hipLaunchKernelGGL(gated_linear_attention_reg_kernel<RP>, grid, dim3(KVA_WAVE), 0, stream, a, y, y_dtype,          \
+                       y_stride, q_off, k_off, v_off, alpha, alpha_stride, q_mul)
+        if (dim <= 64) KVA_GLA_REG(4);
+        else KVA_GLA_REG(8);
+#undef KVA_GLA_REG
+        KVA_CHECK_LAUNCH("gated_linear_attention");
+        return KVA_OK;
+    }
     const int chunk = rec_chunk(dim, 3);
     KVA_REQUIRE(chunk > 0, "gated_linear_attention: key size %d does not fit the LDS", dim);
     RecArgs a{out, state, (size_t)seat_stride, state_off, entry_q_start, entry_seat, heads, heads, dim, vdim, chunk};
     const size_t lds = ((size_t)dim * REC_COLS + (size_t)chunk * dim * 3) * sizeof(float);
     const int slices = (vdim + REC_COLS - 1) / REC_COLS;
     hipLaunchKernelGGL(gated_linear_attention_kernel, dim3(heads * slices, entries), dim3(KVA_WAVE), lds, stream, a, y,
-                       y_dtype, y_stride, q_off, k_off, v_off, z, z_dtype, z_stride, z_off, z_bias, 1.0f / tau, q_mul);
+                       y_dtype, y_stride, q_off, k_off, v_off, alpha, alpha_stride, q_mul);
     KVA_CHECK_LAUNCH("gated_linear_attention");
     return KVA_OK;
 }

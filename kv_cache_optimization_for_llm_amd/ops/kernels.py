@@ -1427,18 +1427,17 @@ def gated_delta_rule(qkv: torch.Tensor, y: torch.Tensor, beta_off: int, decay_of
     return out
 
 
-def gated_linear_attention(y: torch.Tensor, q_off: int, k_off: int, v_off: int, z: torch.Tensor, z_bias: torch.Tensor,
-                           tau: float, q_mul: float, out: torch.Tensor, state: torch.Tensor, state_off: int,
-                           entry_q_start: torch.Tensor, entry_seat: torch.Tensor, heads: int, dim: int,
-                           vdim: int) -> torch.Tensor:
-    """Per head and token, in order: ``S <- diag(alpha) S + k v^T; o = S^T (q_mul q)`` with a decay
-    per key channel ``alpha = sigmoid(z + z_bias)^(1 / tau)``.  q, k (``heads x dim``) and v (``heads x
-    vdim``) are columns of ``y`` from ``q_off``, ``k_off``, ``v_off`` on; ``z`` is ``[T, heads * dim]``.
-    ``out`` fp32 ``[T, heads * vdim]``."""
+def gated_linear_attention(y: torch.Tensor, q_off: int, k_off: int, v_off: int, alpha: torch.Tensor, q_mul: float,
+                           out: torch.Tensor, state: torch.Tensor, state_off: int, entry_q_start: torch.Tensor,
+                           entry_seat: torch.Tensor, heads: int, dim: int, vdim: int) -> torch.Tensor:
+    """Per head and token, in order: ``S <- diag(alpha) S + k v^T; o = S^T (q_mul q)`` with a decay per
+    key channel ``alpha`` (fp32 ``[T, heads * dim]``; :func:`small_product_f32` makes it from a low-rank
+    projection).  q, k (``heads x dim``) and v (``heads x vdim``) are columns of ``y`` from ``q_off``,
+    ``k_off``, ``v_off`` on.  ``out`` fp32 ``[T, heads * vdim]``."""
     tokens = out.shape[0]
     if y.dim() != 2 or y.shape[0] != tokens or out.shape != (tokens, heads * vdim) or out.dtype != torch.float32 \
-            or z.shape != (tokens, heads * dim) or z_bias.shape != (heads * dim,):
-        raise KernelError(f"gated_linear_attention: y {tuple(y.shape)}, z {tuple(z.shape)}, out {tuple(out.shape)} do not fit")
+            or alpha.shape != (tokens, heads * dim) or alpha.dtype != torch.float32:
+        raise KernelError(f"gated_linear_attention: y {tuple(y.shape)}, alpha {tuple(alpha.shape)}, out {tuple(out.shape)} do not fit")
     for off, n in ((q_off, heads * dim), (k_off, heads * dim), (v_off, heads * vdim)):
         if not 0 <= off <= y.shape[1] - n:
             raise KernelError("gated_linear_attention: q, k or v columns lie outside y")
@@ -1446,9 +1445,8 @@ def gated_linear_attention(y: torch.Tensor, q_off: int, k_off: int, v_off: int, 
     qs, seat, entries = _entries((entry_q_start, entry_seat), "gated_linear_attention")
     check(hip_lib().kva_gated_linear_attention(
         _dev(out, "out"), _dev(state, "state"), seat_stride, int(state_off), _dev(y, "y"), dtype_code(y.dtype),
-        y.shape[1], int(q_off), int(k_off), int(v_off), _dev(z, "z"), dtype_code(z.dtype), z.shape[1], 0,
-        _dev(z_bias, "z_bias", torch.float32), float(tau), float(q_mul), qs, seat, entries, heads, dim, vdim,
-        _stream()), "gated_linear_attention")
+        y.shape[1], int(q_off), int(k_off), int(v_off), _dev(alpha, "alpha"), alpha.shape[1], float(q_mul), qs, seat,
+        entries, heads, dim, vdim, _stream()), "gated_linear_attention")
     return out
 
 
@@ -1545,6 +1543,28 @@ def moe_expert_rows(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, sorted_
     return out
 
 
+SMALL_PRODUCT_MAX_K = 8192
+
+
+def small_product_f32(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                      decay_tau: float = 0.0) -> torch.Tensor:
+    """``out = x @ w^T (+ bias)`` with fp32 products, sums and results, for small matrices whose results must
+    not be rounded to 16 bits (a router's logits, the second half of a low-rank projection that makes
+    decays).  With ``decay_tau`` > 0 the result is turned into a decay, ``sigmoid(.)^(1 / decay_tau)``.
+    ``x`` ``[T, K]`` may be columns of a wider buffer; ``x`` and ``w`` ``[N, K]`` are bf16 or fp32."""
+    tokens, k = x.shape
+    if bias is not None and (bias.shape != (w.shape[0],) or bias.dtype != torch.float32):
+        raise KernelError("small_product_f32: the bias is fp32, one value per output")
+    if w.dim() != 2 or w.shape[1] != k or out.shape != (tokens, w.shape[0]) or out.dtype != torch.float32 \
+            or x.stride(1) != 1 or not 0 < k <= SMALL_PRODUCT_MAX_K:
+        raise KernelError(f"small_product_f32: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
+    check(hip_lib().kva_small_product_f32(
+        _dev(out, "out"), _dev(x, "x", contiguous=False), dtype_code(x.dtype), x.stride(0) if tokens > 1 else k,
+        _dev(w, "w"), dtype_code(w.dtype), tokens, w.shape[0], k, _opt(bias, "bias"),
+        1.0 / float(decay_tau) if decay_tau > 0 else 0.0, _stream()), "small_product_f32")
+    return out
+
+
 def moe_combine(x: torch.Tensor, rows: torch.Tensor, idx: torch.Tensor, wgt: torch.Tensor, experts: int,
                 out: torch.Tensor) -> torch.Tensor:
     """``out[t] = sum over the token's choices`` of the slot's row of ``rows`` (fp32 ``[T * top, width]``,
@@ -1579,7 +1599,7 @@ KERNEL_CLASSES = {
     "causal_conv_act": "recurrent mixers", "gated_delta_rule": "recurrent mixers",
     "gated_linear_attention": "recurrent mixers", "head_norm_gate": "elementwise",
     "moe_route": "routed experts", "moe_align": "routed experts", "moe_expert_rows": "routed experts",
-    "moe_combine": "routed experts",
+    "moe_combine": "routed experts", "small_product_f32": "small fp32 products",
 }
 
 

@@ -23,7 +23,6 @@ from ..config.registry import FEED_FORWARDS
 from ..models.spec import TensorSpec
 from ..ops import kernels as K
 from .base import FeedForward, MixerContext
-from .linear import Linear
 
 
 @FEED_FORWARDS.register("routed_experts")
@@ -63,7 +62,7 @@ class RoutedExperts(FeedForward):
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         n = self.names
-        self.router = Linear(tensors[n["router"]].float())          # router logits are formed in 32-bit
+        self.router = tensors[n["router"]].contiguous()             # its logits are formed in 32-bit (ops.kernels.small_product_f32)
         self.correction = tensors[n["correction"]].float().contiguous() if self.has_correction else None
         if self.experts:
             self.w_up = torch.stack([tensors[n["up"].format(e=e)] for e in range(self.experts)]).contiguous()
@@ -76,7 +75,7 @@ class RoutedExperts(FeedForward):
 
     def forward(self, x, ctx: MixerContext, tail=None):
         T, dev = x.shape[0], x.device
-        logits = self.router(x, out_dtype=torch.float32)
+        logits = K.small_product_f32(x, self.router, torch.empty((T, self.outputs), dtype=torch.float32, device=dev))
         idx = torch.empty((T, self.top), dtype=torch.int32, device=dev)
         wgt = torch.empty((T, self.top), dtype=torch.float32, device=dev)
         K.moe_route(logits, self.correction, self.top, idx, wgt, self.renormalise)

@@ -25,7 +25,6 @@ from ..config.registry import MIXERS
 from ..models.spec import TensorSpec
 from ..ops import kernels as K
 from .base import MixerContext, ProjectedMixer
-from .linear import Linear
 
 
 def _names(defaults: Dict[str, str], given: Optional[Dict[str, str]], prefix: str) -> Dict[str, str]:
@@ -76,7 +75,7 @@ class GatedLinearAttention(ProjectedMixer):
         hd, hv = self.num_heads * self.head_dim, self.inner_width
         self.q_off, self.k_off, self.v_off, self.g_off, self.a_off = 0, hd, 2 * hd, 2 * hd + hv, 2 * hd + 2 * hv
         # decays are formed in 32-bit: the second matrix of the low-rank projection multiplies in fp32
-        self.a2 = Linear(t["a2"].float())
+        self.a2 = t["a2"].contiguous()
         self.a2_bias = t["a2_bias"].float().contiguous()
         self.norm_weight = t["norm"].float().contiguous()
         self.load_projections()
@@ -95,12 +94,14 @@ class GatedLinearAttention(ProjectedMixer):
 
     def forward_inner(self, y, col0, ctx: MixerContext, state_off, out, out_col0, mul) -> None:
         batch, T = ctx.batch, y.shape[0]
-        low = y[:, col0 + self.a_off:col0 + self.a_off + self.rank].contiguous()
-        z = self.a2(low, out_dtype=torch.float32)
+        # the decays: the low-rank projection's second half, its bias, sigmoid and power in one 32-bit pass
+        alpha = K.small_product_f32(y[:, col0 + self.a_off:col0 + self.a_off + self.rank], self.a2,
+                                    torch.empty((T, self.num_heads * self.head_dim), dtype=torch.float32, device=y.device),
+                                    bias=self.a2_bias, decay_tau=self.tau)
         o = torch.empty((T, self.inner_width), dtype=torch.float32, device=y.device)
-        K.gated_linear_attention(y, col0 + self.q_off, col0 + self.k_off, col0 + self.v_off, z, self.a2_bias, self.tau,
-                                 self.query_scale, o, ctx.state, state_off, batch.entry_q_start, batch.entry_seat,
-                                 self.num_heads, self.head_dim, self.value_dim)
+        K.gated_linear_attention(y, col0 + self.q_off, col0 + self.k_off, col0 + self.v_off, alpha, self.query_scale, o,
+                                 ctx.state, state_off, batch.entry_q_start, batch.entry_seat, self.num_heads,
+                                 self.head_dim, self.value_dim)
         K.head_norm_gate(o, self.norm_weight, self.norm_eps, y, col0 + self.g_off, out, out_col0, self.num_heads,
                          self.value_dim, "silu", mul)
 

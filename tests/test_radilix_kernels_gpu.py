@@ -192,7 +192,9 @@ def test_gated_linear_attention_over_steps(heads, dim, vdim, portions, gpu):
         ys = torch.cat([y[s][a:a + n] for s, n, a in zip(seats, lens, starts)])
         zs = torch.cat([z[s][a:a + n] for s, n, a in zip(seats, lens, starts)])
         out = torch.empty((ys.shape[0], heads * vdim), dtype=torch.float32, device="cuda")
-        return K.gated_linear_attention(dev(ys), q_off, k_off, v_off, dev(zs), dev(zb), tau, q_mul, out, state, 0,
+        # the decays as the mixer makes them: a small product (here with the unit matrix), bias, sigmoid, power
+        alpha = K.small_product_f32(dev(zs), dev(torch.eye(heads * dim)), torch.empty_like(dev(zs)), bias=dev(zb), decay_tau=tau)
+        return K.gated_linear_attention(dev(ys), q_off, k_off, v_off, alpha, q_mul, out, state, 0,
                                         ints(np.cumsum([0] + lens)), ints(seats), heads, dim, vdim)
     got = run_in_steps(lengths, portions, launch)
     for s, n in lengths.items():
@@ -229,13 +231,13 @@ def test_a_seat_used_again_after_zeroing_forgets_and_a_far_token_is_remembered(g
             K.gated_delta_rule(dev(rows[lo:hi]), dev(y[lo:hi]), 0, 1, dev(torch.zeros(1)), dev(torch.zeros(1)), out[lo:hi],
                                state, 0, ints([0, hi - lo]), ints([1]), 1, 1, dim, vdim)
         torch.testing.assert_close(out[-1].cpu(), v[0] * dim ** -0.5, rtol=1e-4, atol=1e-4)
-    # gated linear attention: alpha = sigmoid(40)^(1/tau) = 1
+    # gated linear attention: alpha = sigmoid(40)^(1/2) = 1
     yy = torch.cat([q, k, v], dim=1)
     z = torch.full((n, dim), 40.0)
     state.zero_()
     for lo in range(0, n, 50):
         hi = min(n, lo + 50)
-        K.gated_linear_attention(dev(yy[lo:hi]), 0, dim, 2 * dim, dev(z[lo:hi]), dev(torch.zeros(dim)), 2.0, 1.0, out[lo:hi],
+        K.gated_linear_attention(dev(yy[lo:hi]), 0, dim, 2 * dim, dev(torch.sigmoid(z[lo:hi]) ** 0.5), 1.0, out[lo:hi],
                                  state, 0, ints([0, hi - lo]), ints([0]), 1, dim, vdim)
     torch.testing.assert_close(out[-1].cpu(), v[0], rtol=1e-5, atol=1e-5)
 
@@ -325,3 +327,17 @@ def test_rotation_of_the_first_elements_with_a_bias_and_the_cache_write(heads, k
         pg, off = int(slots[t]) // page, int(slots[t]) % page
         torch.testing.assert_close(keys[pg, :, off], k[t], **tol)
         torch.testing.assert_close(v_cache[pg, :, :, off].cpu().to(F), v[t], **tol)
+
+
+# ---- small products with 32-bit results ---------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("tokens, n, k", [(1, 18, 320), (9, 5, 72), (33, 192, 16), (4, 300, 6), (7, 3, 2048), (2, 40, 130)])
+def test_small_products_keep_32_bits(tokens, n, k, dtype, gpu):
+    g = torch.Generator().manual_seed(n + k)
+    wide = torch.randn(tokens, k + 13, generator=g).to(dtype)
+    w = torch.randn(n, k, generator=g).to(dtype)
+    buf = dev(wide, dtype)
+    out = torch.empty((tokens, n), dtype=torch.float32, device="cuda")
+    K.small_product_f32(buf[:, 5:5 + k], dev(w, dtype), out)
+    want = wide[:, 5:5 + k].to(F) @ w.to(F).T
+    torch.testing.assert_close(out.cpu().to(F), want, rtol=1e-5, atol=1e-5 * k ** 0.5)
