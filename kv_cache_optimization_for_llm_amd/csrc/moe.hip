@@ -202,58 +202,96 @@ moe_expert_rows_kernel(MoeRows a, void *__restrict__ out, int out_dtype, const T
     }
 }
 
-// matrix cores: a workgroup takes a tile of 16 rows and NT tiles of 16 outputs; out^T[n, t] =
+// matrix cores: a workgroup takes RT tiles of 16 rows and NT tiles of 16 outputs; out^T[n, t] =
 // W[e][n, :] . x[t, :]; operands straight from memory, 16 bytes a lane and product.  Its four
-// wavefronts take a quarter of K each (the same quarters whatever NT and the batch are) and the
+// wavefronts take a quarter of K each (the same quarters whatever NT, RT and the batch are) and the
 // first adds the four partial results up in a fixed order: with few tiles - decoded tokens - there are
-// four times as many wavefronts streaming the experts' matrices.
-template <int NT>
-__global__ void __launch_bounds__(256)
-moe_expert_rows_mfma_kernel(MoeRows a, void *__restrict__ out, int out_dtype, const bf16_t *__restrict__ x,
-                            const bf16_t *__restrict__ w) {
-    __shared__ float red[3][NT][KVA_WAVE][4];
-    const int tile = blockIdx.y, e = a.tile_expert[tile];
-    if (e < 0) return;
+// four times as many wavefronts streaming the experts' matrices.  Row tiles of one expert (the list is
+// sorted by expert, so neighbours mostly are) share what is loaded of its matrix; a group of tiles
+// that spans two experts is walked tile by tile.
+template <int NT, int RT>
+__device__ inline void moe_tiles_product(const MoeRows &a, void *__restrict__ out, int out_dtype,
+                                         const bf16_t *__restrict__ x, const bf16_t *__restrict__ w, int first_tile,
+                                         int e, int n_first, float (*red)[KVA_WAVE][4]) {
     const int lane = threadIdx.x % KVA_WAVE, wave = threadIdx.x / KVA_WAVE, r = lane & 15, g = lane >> 4;
-    const int n_first = blockIdx.x * 16 * NT;
-    const int place = tile * MOE_TILE + r, slot = a.sorted_slot[place];
-    const size_t src = a.mode == 0 ? (size_t)(slot < 0 ? 0 : slot / a.top) : (size_t)place;
-    const bf16_t *xrow = x + src * a.K + 8 * g;
+    int place[RT], slot[RT];
+    const bf16_t *xrow[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        place[rt] = (first_tile + rt) * MOE_TILE + r;
+        slot[rt] = a.sorted_slot[place[rt]];
+        const size_t src = a.mode == 0 ? (size_t)(slot[rt] < 0 ? 0 : slot[rt] / a.top) : (size_t)place[rt];
+        xrow[rt] = x + src * a.K + 8 * g;
+    }
     const bf16_t *wrow[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
         wrow[nt] = w + ((size_t)e * a.N + min(n_first + 16 * nt + r, a.N - 1)) * a.K + 8 * g;
-    f32x4 acc[NT];
+    f32x4 acc[NT][RT];
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) acc[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) acc[nt][rt] = f32x4{0.f, 0.f, 0.f, 0.f};
     const int steps = a.K / 32, per = (steps + 3) / 4;
     const int s0 = wave * per, s1 = min(steps, s0 + per);
-#pragma unroll 4
+#pragma unroll 2
     for (int s = s0; s < s1; ++s) {
         const int k0 = 32 * s;
-        Frag8 xf, wf[NT];
-        xf.u4 = *reinterpret_cast<const uint4 *>(xrow + k0);
+        Frag8 xf[RT], wf[NT];
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) xf[rt].u4 = *reinterpret_cast<const uint4 *>(xrow[rt] + k0);
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) wf[nt].u4 = *reinterpret_cast<const uint4 *>(wrow[nt] + k0);
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[nt].v, xf.v, acc[nt], 0, 0, 0);
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+                acc[nt][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[nt].v, xf[rt].v, acc[nt][rt], 0, 0, 0);
     }
+    __syncthreads();                 // whoever still reads the partial results of the call before is done
     if (wave > 0)
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) red[wave - 1][nt][lane][i] = acc[nt][i];
+            for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) red[((wave - 1) * NT + nt) * RT + rt][lane][i] = acc[nt][rt][i];
     __syncthreads();
-    if (wave > 0 || slot < 0) return;
+    if (wave > 0) return;
     // lane (row r, group g) holds outputs n0 + 4 g .. + 3 of its row
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
+    for (int rt = 0; rt < RT; ++rt) {
+        if (slot[rt] < 0) continue;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int n = n_first + 16 * nt + 4 * g + i;
-            const float v = ((acc[nt][i] + red[0][nt][lane][i]) + red[1][nt][lane][i]) + red[2][nt][lane][i];
-            if (n < a.N) moe_store(a, out, out_dtype, place, slot, n, v);
-        }
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int n = n_first + 16 * nt + 4 * g + i;
+                const float v = ((acc[nt][rt][i] + red[(0 * NT + nt) * RT + rt][lane][i]) + red[(1 * NT + nt) * RT + rt][lane][i])
+                                + red[(2 * NT + nt) * RT + rt][lane][i];
+                if (n < a.N) moe_store(a, out, out_dtype, place[rt], slot[rt], n, v);
+            }
+    }
+}
+
+template <int NT, int RT>
+__global__ void __launch_bounds__(256)
+moe_expert_rows_mfma_kernel(MoeRows a, void *__restrict__ out, int out_dtype, const bf16_t *__restrict__ x,
+                            const bf16_t *__restrict__ w, int max_tiles) {
+    __shared__ float red[3 * NT * RT][KVA_WAVE][4];
+    const int first = blockIdx.y * RT, n_first = blockIdx.x * 16 * NT;
+    const int e0 = a.tile_expert[first];
+    bool same = e0 >= 0;
+#pragma unroll
+    for (int rt = 1; rt < RT; ++rt) same = same && first + rt < max_tiles && a.tile_expert[first + rt] == e0;
+    if (same) {
+        moe_tiles_product<NT, RT>(a, out, out_dtype, x, w, first, e0, n_first, red);
+        return;
+    }
+    for (int rt = 0; rt < RT; ++rt) {
+        const int e = first + rt < max_tiles ? a.tile_expert[first + rt] : -1;
+        if (e >= 0) moe_tiles_product<NT, 1>(a, out, out_dtype, x, w, first + rt, e, n_first, red);
+    }
 }
 
 extern "C" int kva_moe_expert_rows(void *out, int out_dtype, const void *x, const void *w, int dtype,
@@ -268,13 +306,14 @@ extern "C" int kva_moe_expert_rows(void *out, int out_dtype, const void *x, cons
     if (max_tiles == 0) return KVA_OK;
     MoeRows a{sorted_slot, tile_expert, slot_weight, top, N, K, mode, act};
     if (dtype == KVA_BF16 && K % 32 == 0) {
-        // few tiles: 16 outputs a workgroup, so that enough of them stream the matrices; many: 64, which share x
+        // few tiles: 16 outputs a workgroup, so that enough of them stream the matrices; many: 64 outputs and
+        // four row tiles, which share what they load
         if ((long long)max_tiles * ((N + 15) / 16) <= 8192)
-            hipLaunchKernelGGL(moe_expert_rows_mfma_kernel<1>, dim3((N + 15) / 16, max_tiles), dim3(256), 0, stream, a,
-                               out, out_dtype, (const bf16_t *)x, (const bf16_t *)w);
+            hipLaunchKernelGGL((moe_expert_rows_mfma_kernel<1, 1>), dim3((N + 15) / 16, max_tiles), dim3(256), 0, stream, a,
+                               out, out_dtype, (const bf16_t *)x, (const bf16_t *)w, max_tiles);
         else
-            hipLaunchKernelGGL(moe_expert_rows_mfma_kernel<4>, dim3((N + 63) / 64, max_tiles), dim3(256), 0, stream, a,
-                               out, out_dtype, (const bf16_t *)x, (const bf16_t *)w);
+            hipLaunchKernelGGL((moe_expert_rows_mfma_kernel<4, 4>), dim3((N + 63) / 64, (max_tiles + 3) / 4), dim3(256), 0,
+                               stream, a, out, out_dtype, (const bf16_t *)x, (const bf16_t *)w, max_tiles);
     } else if (dtype == KVA_BF16) {
         hipLaunchKernelGGL(moe_expert_rows_kernel<bf16_t>, dim3((N + 63) / 64, max_tiles), dim3(256), 0, stream, a, out,
                            out_dtype, (const bf16_t *)x, (const bf16_t *)w);

@@ -10,11 +10,11 @@
 //    weight, times act(gate), times a constant, into a column range of a wider buffer.
 //
 // The state S [key channels, value channels] of a (request, head) is fp32 and lives in the seat's
-// state row between steps.  A wavefront takes 16 value columns of one head: lane = 16 * r + c owns
-// the rows i = r, r + 4, ... of column c, kept in LDS while the step's tokens of the request are
-// walked in order; sums over rows are finished between the four lanes of a column.  Columns are
-// independent of each other in both recurrences, so a head's columns go to different wavefronts.
-// The order of every sum depends on the sizes alone: a token's result is the same bit for bit
+// state row between steps.  Columns are independent of each other in both recurrences, so a head's
+// columns go to different wavefronts, which walk the step's tokens of the request in order.  Key sizes
+// up to 128 keep their part of S in registers (4 columns a wavefront, 16 lanes a column); larger
+// ones keep it in LDS (16 columns a wavefront, lane = 16 r + c owns the rows r, r + 4, ... of column
+// c).  The order of every sum depends on the sizes alone: a token's result is the same bit for bit
 // however the request's tokens were cut into steps and whatever else the step holds.
 #include "common.h"
 #include <math.h>
@@ -250,30 +250,35 @@ gated_linear_attention_kernel(RecArgs a, const void *__restrict__ y, int y_dtype
 }
 
 // ---- the two recurrences with the state in registers (key sizes up to 128) ----------------------
-// A wavefront takes 4 value columns of a head; the 16 lanes of a row of the wavefront share a
-// column.  Lane (c, r) owns, of column c, the rows 4 (16 j + r) .. + 3 for j < RP / 4 in RP
-// registers (rows from `dim` on are padding and stay zero): a 16-byte LDS read per j and lane takes
-// 256 neighbouring bytes of a token's k, q or alpha, and a sum over the rows ends with four
-// rotations inside the lanes' row.  A chunk of 16 tokens is staged in LDS - q, k (and the decays)
-// padded to 16 RP elements a token, the 4 values of the wavefront's columns, the token's two numbers;
-// the next chunk's global loads are issued before the current one is walked.  A head's columns are
-// spread over vdim / 4 wavefronts: a prompt of one request fills the chip at the sizes of a model.
+// A workgroup of four wavefronts takes 16 value columns of a head, a wavefront 4 of them; the 16
+// lanes of a row of the wavefront share a column.  Lane (c, r) owns, of column c, the rows
+// 4 (16 j + r) .. + 3 for j < RP / 4 in RP registers (rows from `dim` on are padding and stay zero): a
+// 16-byte LDS read per j and lane takes 256 neighbouring bytes of a token's k, q or alpha, and a sum
+// over the rows ends with four rotations inside the lanes' row.  A chunk of 16 tokens is staged in
+// LDS once for the four wavefronts - q, k (and the decays) padded to 16 RP elements a token, the 16
+// values of the workgroup's columns, the token's numbers; the next chunk's global loads are issued
+// before the current one is walked, and no wavefront waits for another inside a chunk.
 #define REC_CHUNK 16
-#define REG_COLS 4
+#define REG_COLS 4           // columns a wavefront
 #define REG_LANES 16         // lanes that share a column
+#define REG_WAVES 4
+#define REG_BLOCK_COLS (REG_COLS * REG_WAVES)
+#define REG_THREADS (KVA_WAVE * REG_WAVES)
 
 template <int RP>
-__global__ void __launch_bounds__(KVA_WAVE)
+__global__ void __launch_bounds__(REG_THREADS)
 gated_delta_rule_reg_kernel(RecArgs a, const float *__restrict__ qkv, int conv_stride, const void *__restrict__ y,
                             int y_dtype, int y_stride, int beta_off, int decay_off, const float *__restrict__ a_log,
                             const float *__restrict__ dt_bias, float unit_eps) {
-    constexpr int DP = REG_LANES * RP, DS = DP + 4, CH = REC_CHUNK, PER = CH * DP / KVA_WAVE;   // token rows 4 banks apart
+    constexpr int DP = REG_LANES * RP, DS = DP + 4, CH = REC_CHUNK, PER = CH * DP / REG_THREADS;   // token rows 4 banks apart
     __shared__ __attribute__((aligned(16))) float qs[CH * DS];
     __shared__ __attribute__((aligned(16))) float ks[CH * DS];
-    __shared__ float vs[CH * REG_COLS], bs[CH], gs[CH], nq[CH], nk[CH];
-    const int lane = threadIdx.x, c = lane / REG_LANES, r = lane % REG_LANES;
-    const int slices = (a.vdim + REG_COLS - 1) / REG_COLS;
-    const int head = blockIdx.x / slices, col0 = (blockIdx.x % slices) * REG_COLS, col = col0 + c;
+    __shared__ float vs[CH * REG_BLOCK_COLS], bs[CH], gs[CH], nq[CH], nk[CH];
+    const int tid = threadIdx.x, lane = tid % KVA_WAVE, wave = tid / KVA_WAVE;
+    const int c = lane / REG_LANES, r = lane % REG_LANES;
+    const int slices = (a.vdim + REG_BLOCK_COLS - 1) / REG_BLOCK_COLS;
+    const int head = blockIdx.x / slices, block_col0 = (blockIdx.x % slices) * REG_BLOCK_COLS;
+    const int col = block_col0 + wave * REG_COLS + c;
     const int e = blockIdx.y;
     const int q0 = a.entry_q_start[e], n = a.entry_q_start[e + 1] - q0;
     if (n <= 0) return;
@@ -293,19 +298,20 @@ gated_delta_rule_reg_kernel(RecArgs a, const float *__restrict__ qkv, int conv_s
 #pragma unroll
         for (int j = 0; j < PER; ++j) {
             pq[j] = pk[j] = 0.f;
-            if (KVA_WAVE * j / DP >= m) continue;           // (the whole wavefront: a decoded token loads one row)
-            const int x = lane + KVA_WAVE * j, tt = x / DP, i = x % DP;
-            if (i >= d) continue;
+            if (REG_THREADS * j / DP >= m) continue;        // (the whole workgroup: a decoded token loads one row)
+            const int x = tid + REG_THREADS * j, tt = x / DP, i = x % DP;
+            if (tt >= m || i >= d) continue;
             const size_t row = (size_t)(q0 + t0 + tt) * conv_stride;
             pq[j] = qkv[row + kvh * d + i];
             pk[j] = qkv[row + k_col + kvh * d + i];
         }
-        {   // 16 tokens x 4 columns: one value a lane
-            const int tt = lane / REG_COLS, cc = lane % REG_COLS;
-            pv = (tt < m && col0 + cc < dv) ? qkv[(size_t)(q0 + t0 + tt) * conv_stride + v_col + head * dv + col0 + cc] : 0.f;
+        {   // 16 tokens x 16 columns: one value a thread
+            const int tt = tid / REG_BLOCK_COLS, cc = tid % REG_BLOCK_COLS;
+            pv = (tt < m && block_col0 + cc < dv)
+                     ? qkv[(size_t)(q0 + t0 + tt) * conv_stride + v_col + head * dv + block_col0 + cc] : 0.f;
         }
-        if (lane < m) {
-            const size_t yrow = (size_t)(q0 + t0 + lane) * y_stride;
+        if (tid < m) {
+            const size_t yrow = (size_t)(q0 + t0 + tid) * y_stride;
             pb = rec_ld(y, y_dtype, yrow + beta_off + head);
             pg = rec_ld(y, y_dtype, yrow + decay_off + head);
         }
@@ -316,17 +322,17 @@ gated_delta_rule_reg_kernel(RecArgs a, const float *__restrict__ qkv, int conv_s
         __syncthreads();
 #pragma unroll
         for (int j = 0; j < PER; ++j) {
-            const int x = lane + KVA_WAVE * j, at = (x / DP) * DS + x % DP;
+            const int x = tid + REG_THREADS * j, at = (x / DP) * DS + x % DP;
             qs[at] = pq[j];
             ks[at] = pk[j];
         }
-        vs[lane] = pv;
-        if (lane < m) {
-            bs[lane] = rec_sigmoid(pb);
-            gs[lane] = expf(-rate * rec_softplus(pg + bias));
+        vs[tid] = pv;
+        if (tid < m) {
+            bs[tid] = rec_sigmoid(pb);
+            gs[tid] = expf(-rate * rec_softplus(pg + bias));
         }
         __syncthreads();
-        {   // what makes q and k unit vectors: token tt by the four lanes 4 tt .. 4 tt + 3, every fourth element each
+        if (wave == 0) {   // what makes q and k unit vectors: token tt by the four lanes 4 tt .. 4 tt + 3, every fourth element each
             const int tt = lane / 4, part = lane % 4;
             float sq = 0.f, sk = 0.f;
             if (tt < m)
@@ -346,7 +352,7 @@ gated_delta_rule_reg_kernel(RecArgs a, const float *__restrict__ qkv, int conv_s
         for (int tt = 0; tt < m; ++tt) {
             const float4 *k4 = reinterpret_cast<const float4 *>(ks + tt * DS) + r;
             const float4 *q4 = reinterpret_cast<const float4 *>(qs + tt * DS) + r;
-            const float g = gs[tt], beta = bs[tt], v = vs[tt * REG_COLS + c], mq = nq[tt], mk = nk[tt];
+            const float g = gs[tt], beta = bs[tt], v = vs[tt * REG_BLOCK_COLS + wave * REG_COLS + c], mq = nq[tt], mk = nk[tt];
             // the unit vectors' factors multiply the sums: S^T (mk k) = mk (S^T k), S^T (mq q) likewise
             float4 kk[RP / 4];
             float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
@@ -387,17 +393,19 @@ gated_delta_rule_reg_kernel(RecArgs a, const float *__restrict__ qkv, int conv_s
 }
 
 template <int RP>
-__global__ void __launch_bounds__(KVA_WAVE)
+__global__ void __launch_bounds__(REG_THREADS)
 gated_linear_attention_reg_kernel(RecArgs a, const void *__restrict__ y, int y_dtype, int y_stride, int q_off, int k_off,
                                   int v_off, const float *__restrict__ alpha, int alpha_stride, float q_mul) {
-    constexpr int DP = REG_LANES * RP, DS = DP + 4, CH = REC_CHUNK, PER = CH * DP / KVA_WAVE;   // token rows 4 banks apart
+    constexpr int DP = REG_LANES * RP, DS = DP + 4, CH = REC_CHUNK, PER = CH * DP / REG_THREADS;   // token rows 4 banks apart
     __shared__ __attribute__((aligned(16))) float qs[CH * DS];
     __shared__ __attribute__((aligned(16))) float ks[CH * DS];
     __shared__ __attribute__((aligned(16))) float as[CH * DS];
-    __shared__ float vs[CH * REG_COLS];
-    const int lane = threadIdx.x, c = lane / REG_LANES, r = lane % REG_LANES;
-    const int slices = (a.vdim + REG_COLS - 1) / REG_COLS;
-    const int head = blockIdx.x / slices, col0 = (blockIdx.x % slices) * REG_COLS, col = col0 + c;
+    __shared__ float vs[CH * REG_BLOCK_COLS];
+    const int tid = threadIdx.x, lane = tid % KVA_WAVE, wave = tid / KVA_WAVE;
+    const int c = lane / REG_LANES, r = lane % REG_LANES;
+    const int slices = (a.vdim + REG_BLOCK_COLS - 1) / REG_BLOCK_COLS;
+    const int head = blockIdx.x / slices, block_col0 = (blockIdx.x % slices) * REG_BLOCK_COLS;
+    const int col = block_col0 + wave * REG_COLS + c;
     const int e = blockIdx.y;
     const int q0 = a.entry_q_start[e], n = a.entry_q_start[e + 1] - q0;
     if (n <= 0) return;
@@ -415,16 +423,17 @@ gated_linear_attention_reg_kernel(RecArgs a, const void *__restrict__ y, int y_d
 #pragma unroll
         for (int j = 0; j < PER; ++j) {
             pq[j] = pk[j] = pa[j] = 0.f;
-            if (KVA_WAVE * j / DP >= m) continue;           // (the whole wavefront: a decoded token loads one row)
-            const int x = lane + KVA_WAVE * j, tt = x / DP, i = x % DP;
-            if (i >= d) continue;
+            if (REG_THREADS * j / DP >= m) continue;        // (the whole workgroup: a decoded token loads one row)
+            const int x = tid + REG_THREADS * j, tt = x / DP, i = x % DP;
+            if (tt >= m || i >= d) continue;
             const size_t row = (size_t)(q0 + t0 + tt);
             pq[j] = rec_ld(y, y_dtype, row * y_stride + q_off + head * d + i);
             pk[j] = rec_ld(y, y_dtype, row * y_stride + k_off + head * d + i);
             pa[j] = alpha[row * alpha_stride + head * d + i];
         }
-        const int tt = lane / REG_COLS, cc = lane % REG_COLS;
-        pv = (tt < m && col0 + cc < dv) ? rec_ld(y, y_dtype, (size_t)(q0 + t0 + tt) * y_stride + v_off + head * dv + col0 + cc) : 0.f;
+        const int tt = tid / REG_BLOCK_COLS, cc = tid % REG_BLOCK_COLS;
+        pv = (tt < m && block_col0 + cc < dv)
+                 ? rec_ld(y, y_dtype, (size_t)(q0 + t0 + tt) * y_stride + v_off + head * dv + block_col0 + cc) : 0.f;
     };
     fetch(0, min(CH, n));
     for (int t0 = 0; t0 < n; t0 += CH) {
@@ -432,19 +441,19 @@ gated_linear_attention_reg_kernel(RecArgs a, const void *__restrict__ y, int y_d
         __syncthreads();
 #pragma unroll
         for (int j = 0; j < PER; ++j) {
-            const int x = lane + KVA_WAVE * j, at = (x / DP) * DS + x % DP;
+            const int x = tid + REG_THREADS * j, at = (x / DP) * DS + x % DP;
             qs[at] = pq[j] * q_mul;
             ks[at] = pk[j];
             as[at] = pa[j];
         }
-        vs[lane] = pv;
+        vs[tid] = pv;
         __syncthreads();
         if (t0 + CH < n) fetch(t0 + CH, min(CH, n - t0 - CH));
         for (int tt = 0; tt < m; ++tt) {
             const float4 *k4 = reinterpret_cast<const float4 *>(ks + tt * DS) + r;
             const float4 *q4 = reinterpret_cast<const float4 *>(qs + tt * DS) + r;
             const float4 *a4 = reinterpret_cast<const float4 *>(as + tt * DS) + r;
-            const float v = vs[tt * REG_COLS + c];
+            const float v = vs[tt * REG_BLOCK_COLS + wave * REG_COLS + c];
             float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
 #pragma unroll
             for (int j = 0; j < RP / 4; ++j) {
@@ -497,9 +506,9 @@ extern "C" int kva_gated_delta_rule(float *out, float *state, long long seat_str
     if (entries == 0) return KVA_OK;
     if (dim <= 128) {
         RecArgs a{out, state, (size_t)seat_stride, state_off, entry_q_start, entry_seat, heads, kv_heads, dim, vdim, REC_CHUNK};
-        const dim3 grid(heads * ((vdim + REG_COLS - 1) / REG_COLS), entries);
+        const dim3 grid(heads * ((vdim + REG_BLOCK_COLS - 1) / REG_BLOCK_COLS), entries);
 #define KVA_DELTA_REG(RP)                                                                                              \
-    hipLaunchKernelGGL(gated_delta_rule_reg_kernel<RP>, grid, dim3(KVA_WAVE), 0, stream, a, qkv, conv_stride, y,       \
+    hipLaunchKernelGGL(gated_delta_rule_reg_kernel<RP>, grid, dim3(REG_THREADS), 0, stream, a, qkv, conv_stride, y,       \
                        y_dtype, y_stride, beta_off, decay_off, a_log, dt_bias, unit_eps)
         if (dim <= 64) KVA_DELTA_REG(4);
         else KVA_DELTA_REG(8);
@@ -528,9 +537,9 @@ extern "C" int kva_gated_linear_attention(float *out, float *state, long long se
     if (entries == 0) return KVA_OK;
     if (dim <= 128) {
         RecArgs a{out, state, (size_t)seat_stride, state_off, entry_q_start, entry_seat, heads, heads, dim, vdim, REC_CHUNK};
-        const dim3 grid(heads * ((vdim + REG_COLS - 1) / REG_COLS), entries);
+        const dim3 grid(heads * ((vdim + REG_BLOCK_COLS - 1) / REG_BLOCK_COLS), entries);
 #define KVA_GLA_REG(RP)                                                                                                \
-    hipLaunchKernelGGL(gated_linear_attention_reg_kernel<RP>, grid, dim3(KVA_WAVE), 0, stream, a, y, y_dtype,          \
+    hipLaunchKernelGGL(gated_linear_attention_reg_kernel<RP>, grid, dim3(REG_THREADS), 0, stream, a, y, y_dtype,          \
                        y_stride, q_off, k_off, v_off, alpha, alpha_stride, q_mul)
         if (dim <= 64) KVA_GLA_REG(4);
         else KVA_GLA_REG(8);

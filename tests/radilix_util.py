@@ -58,7 +58,12 @@ _C1 = gla_layer(4, 64, 64, 16.0, 16, moe(6, 2, 96, identity=1))
 CFG_C = {"architecture": "Radilix", "vocab": 257, "width": 256, "norm": {"eps": 0.02}, "residual_mult": 0.7, "layers": [
     _C0, _C1, parallel_layer((4, 4, 64, 32, 64, 7000.0, 0.11), (2, 1, 32, 128, 2), 0.9, 0.9, moe(4, 1, 64, identity=1)),
     shared(_C1, 1), shared(_C0, 0)]}
-CONFIGS = {"A": (CFG_A, 5), "B": (CFG_B, 6), "C": (CFG_C, 7)}
+# D: no layer keeps keys and values (the cache manager has no paged group); keys of 160 channels (the
+#    recurrences' kernels that keep the state in LDS) and a single expert beside a single identity expert.
+_D0 = gla_layer(2, 160, 24, 5.0, 4, moe(1, 1, 32, identity=1))
+CFG_D = {"architecture": "Radilix", "vocab": 131, "width": 64, "norm": {"eps": 0.05}, "residual_mult": 1.3, "layers": [
+    _D0, gla_layer(4, 12, 12, 1.0, 2), shared(_D0, 0)]}
+CONFIGS = {"A": (CFG_A, 5), "B": (CFG_B, 6), "C": (CFG_C, 7), "D": (CFG_D, 8)}
 
 
 def write_model(folder: str, cfg: dict, seed: int, gain: float = 1.0, edit=None) -> Tuple[str, Dict[str, torch.Tensor]]:

@@ -34,7 +34,7 @@ def engine_for(folder, dtype, **kw):
     return Engine(folder, EngineOptions(**opts))
 
 
-REQUESTS = {"A": [1, 2, 9, 40, 77], "B": [3, 33, 70], "C": [1, 5, 47, 150]}
+REQUESTS = {"A": [1, 2, 9, 40, 77], "B": [3, 33, 70], "C": [1, 5, 47, 150], "D": [2, 35, 64]}
 
 
 def requests_for(name, cfg):
@@ -49,7 +49,7 @@ def check(eng, cfg, state, reqs, steps, dtype, what):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_whole_prompts_and_the_first_tokens(name, dtype, models, gpu):
     cfg, folder, state = models[name]
     reqs = requests_for(name, cfg)
@@ -60,7 +60,7 @@ def test_whole_prompts_and_the_first_tokens(name, dtype, models, gpu):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_prefill_against_token_by_token_decoding(name, dtype, models, gpu):
     """Most of a request in one step, the rest one token at a time (the states and the convolutions'
     last inputs are carried from step to step); and a request decoded from its very first token on."""
@@ -83,7 +83,7 @@ def test_portions_of_any_size(name, sizes, dtype, models, gpu):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name, seed", [("A", 0), ("B", 1), ("B", 2), ("C", 3), ("C", 4)])
+@pytest.mark.parametrize("name, seed", [("A", 0), ("B", 1), ("B", 2), ("C", 3), ("C", 4), ("D", 5)])
 def test_mixed_batches_on_a_small_pool_reuse_pages_and_seats(name, seed, dtype, models, gpu):
     cfg, folder, state = models[name]
     lengths = [40, 3, 90, 25, 61, 2, 130, 47, 33]
@@ -94,7 +94,7 @@ def test_mixed_batches_on_a_small_pool_reuse_pages_and_seats(name, seed, dtype, 
     rows = check(eng, cfg, state, reqs, steps, dtype, "mixed")
     assert len(rows) == sum(lengths)
     stats = eng.cache.stats()
-    assert stats["pages_reused"] > 0 and stats["running"] == 0
+    assert (stats["pages_reused"] > 0 or not eng.cache.groups) and stats["running"] == 0
     assert all(g.free_pages() == g.num_pages for g in eng.cache.groups)
 
 

@@ -140,7 +140,7 @@ def run_in_steps(lengths, portions_of, launch):
     return {s: torch.cat(v) for s, v in got.items()}
 
 
-@pytest.mark.parametrize("heads, kv_heads, dim, vdim", [(2, 1, 32, 32), (4, 2, 16, 24), (3, 3, 20, 7), (2, 2, 128, 48), (6, 2, 8, 70)])
+@pytest.mark.parametrize("heads, kv_heads, dim, vdim", [(2, 1, 32, 32), (4, 2, 16, 24), (3, 3, 20, 7), (2, 2, 128, 48), (6, 2, 8, 70), (2, 1, 160, 20), (1, 1, 64, 3)])
 @pytest.mark.parametrize("portions", [(1000,), (1,), (2, 1, 17, 5, 64)])
 def test_gated_delta_rule_over_steps(heads, kv_heads, dim, vdim, portions, gpu):
     g = torch.Generator().manual_seed(heads * dim + vdim)
@@ -176,7 +176,7 @@ def test_gated_delta_rule_over_steps(heads, kv_heads, dim, vdim, portions, gpu):
     assert (state[:, :4] == 0).all()
 
 
-@pytest.mark.parametrize("heads, dim, vdim", [(4, 48, 32), (1, 16, 16), (3, 20, 9), (2, 128, 40), (5, 8, 64)])
+@pytest.mark.parametrize("heads, dim, vdim", [(4, 48, 32), (1, 16, 16), (3, 20, 9), (2, 128, 40), (5, 8, 64), (2, 144, 18), (1, 100, 5)])
 @pytest.mark.parametrize("portions", [(1000,), (1,), (3, 1, 16, 2, 50)])
 def test_gated_linear_attention_over_steps(heads, dim, vdim, portions, gpu):
     g = torch.Generator().manual_seed(heads * dim + vdim + 1)
