@@ -254,11 +254,11 @@ gated_linear_attention_kernel(RecArgs a, const void *__restrict__ y, int y_dtype
 // lanes of a row of the wavefront share a column.  Lane (c, r) owns, of column c, the rows
 // 4 (16 j + r) .. + 3 for j < RP / 4 in RP registers (rows from `dim` on are padding and stay zero): a
 // 16-byte LDS read per j and lane takes 256 neighbouring bytes of a token's k, q or alpha, and a sum
-// over the rows ends with four rotations inside the lanes' row.  A chunk of 16 tokens is staged in
+// over the rows ends with four rotations inside the lanes' row.  A chunk of 32 tokens is staged in
 // LDS once for the four wavefronts - q, k (and the decays) padded to 16 RP elements a token, the 16
 // values of the workgroup's columns, the token's numbers; the next chunk's global loads are issued
 // before the current one is walked, and no wavefront waits for another inside a chunk.
-#define REC_CHUNK 16
+#define REC_CHUNK 32         // tokens staged at a time: their walk hides the next chunk's trip to memory
 #define REG_COLS 4           // columns a wavefront
 #define REG_LANES 16         // lanes that share a column
 #define REG_WAVES 4
@@ -273,7 +273,7 @@ gated_delta_rule_reg_kernel(RecArgs a, const float *__restrict__ qkv, int conv_s
     constexpr int DP = REG_LANES * RP, DS = DP + 4, CH = REC_CHUNK, PER = CH * DP / REG_THREADS;   // token rows 4 banks apart
     __shared__ __attribute__((aligned(16))) float qs[CH * DS];
     __shared__ __attribute__((aligned(16))) float ks[CH * DS];
-    __shared__ float vs[CH * REG_BLOCK_COLS], bs[CH], gs[CH], nq[CH], nk[CH];
+    __shared__ float vs[CH * REG_BLOCK_COLS], os[CH * REG_BLOCK_COLS], bs[CH], gs[CH], nq[CH], nk[CH];
     const int tid = threadIdx.x, lane = tid % KVA_WAVE, wave = tid / KVA_WAVE;
     const int c = lane / REG_LANES, r = lane % REG_LANES;
     const int slices = (a.vdim + REG_BLOCK_COLS - 1) / REG_BLOCK_COLS;
@@ -293,7 +293,8 @@ gated_delta_rule_reg_kernel(RecArgs a, const float *__restrict__ qkv, int conv_s
     }
     const int k_col = a.kv_heads * d, v_col = 2 * a.kv_heads * d;
     const float rate = expf(a_log[head]), bias = dt_bias[head], q_mul = 1.0f / sqrtf((float)d);
-    float pq[PER], pk[PER], pv = 0.f, pb = 0.f, pg = 0.f;
+    constexpr int VPER = CH * REG_BLOCK_COLS / REG_THREADS;
+    float pq[PER], pk[PER], pv[VPER], pb = 0.f, pg = 0.f;
     auto fetch = [&](int t0, int m) {
 #pragma unroll
         for (int j = 0; j < PER; ++j) {
@@ -305,10 +306,11 @@ gated_delta_rule_reg_kernel(RecArgs a, const float *__restrict__ qkv, int conv_s
             pq[j] = qkv[row + kvh * d + i];
             pk[j] = qkv[row + k_col + kvh * d + i];
         }
-        {   // 16 tokens x 16 columns: one value a thread
-            const int tt = tid / REG_BLOCK_COLS, cc = tid % REG_BLOCK_COLS;
-            pv = (tt < m && block_col0 + cc < dv)
-                     ? qkv[(size_t)(q0 + t0 + tt) * conv_stride + v_col + head * dv + block_col0 + cc] : 0.f;
+#pragma unroll
+        for (int j = 0; j < VPER; ++j) {   // the chunk's tokens x 16 columns
+            const int x = tid + REG_THREADS * j, tt = x / REG_BLOCK_COLS, cc = x % REG_BLOCK_COLS;
+            pv[j] = (tt < m && block_col0 + cc < dv)
+                        ? qkv[(size_t)(q0 + t0 + tt) * conv_stride + v_col + head * dv + block_col0 + cc] : 0.f;
         }
         if (tid < m) {
             const size_t yrow = (size_t)(q0 + t0 + tid) * y_stride;
@@ -326,14 +328,15 @@ gated_delta_rule_reg_kernel(RecArgs a, const float *__restrict__ qkv, int conv_s
             qs[at] = pq[j];
             ks[at] = pk[j];
         }
-        vs[tid] = pv;
+#pragma unroll
+        for (int j = 0; j < VPER; ++j) vs[tid + REG_THREADS * j] = pv[j];
         if (tid < m) {
             bs[tid] = rec_sigmoid(pb);
             gs[tid] = expf(-rate * rec_softplus(pg + bias));
         }
         __syncthreads();
-        if (wave == 0) {   // what makes q and k unit vectors: token tt by the four lanes 4 tt .. 4 tt + 3, every fourth element each
-            const int tt = lane / 4, part = lane % 4;
+        if (wave < CH / 16) {   // what makes q and k unit vectors: a token by four lanes, every fourth element each
+            const int tt = wave * 16 + lane / 4, part = lane % 4;
             float sq = 0.f, sk = 0.f;
             if (tt < m)
                 for (int i = part; i < DP; i += 4) {
@@ -349,16 +352,35 @@ gated_delta_rule_reg_kernel(RecArgs a, const float *__restrict__ qkv, int conv_s
         }
         __syncthreads();
         if (t0 + CH < n) fetch(t0 + CH, min(CH, n - t0 - CH));
-        for (int tt = 0; tt < m; ++tt) {
+        // a token's operands are read from LDS into registers while the token before it is worked on
+        float4 kn[RP / 4], qn[RP / 4];
+        float gn, betan, vn, mqn, mkn;
+        auto read_token = [&](int tt) {
             const float4 *k4 = reinterpret_cast<const float4 *>(ks + tt * DS) + r;
             const float4 *q4 = reinterpret_cast<const float4 *>(qs + tt * DS) + r;
-            const float g = gs[tt], beta = bs[tt], v = vs[tt * REG_BLOCK_COLS + wave * REG_COLS + c], mq = nq[tt], mk = nk[tt];
+#pragma unroll
+            for (int j = 0; j < RP / 4; ++j) {
+                kn[j] = k4[REG_LANES * j];
+                qn[j] = q4[REG_LANES * j];
+            }
+            gn = gs[tt]; betan = bs[tt]; vn = vs[tt * REG_BLOCK_COLS + wave * REG_COLS + c]; mqn = nq[tt]; mkn = nk[tt];
+        };
+        read_token(0);
+        // (unrolled: a token's sums over the rows and its write overlap the next token's update of S)
+#pragma unroll 4
+        for (int tt = 0; tt < m; ++tt) {
+            float4 kk[RP / 4], qq[RP / 4];
+            const float g = gn, beta = betan, v = vn, mq = mqn, mk = mkn;
+#pragma unroll
+            for (int j = 0; j < RP / 4; ++j) {
+                kk[j] = kn[j];
+                qq[j] = qn[j];
+            }
+            read_token(min(tt + 1, CH - 1));
             // the unit vectors' factors multiply the sums: S^T (mk k) = mk (S^T k), S^T (mq q) likewise
-            float4 kk[RP / 4];
             float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
 #pragma unroll
             for (int j = 0; j < RP / 4; ++j) {
-                kk[j] = k4[REG_LANES * j];
                 kk[j].x *= mk; kk[j].y *= mk; kk[j].z *= mk; kk[j].w *= mk;
                 d0 += S[4 * j] * kk[j].x;
                 d1 += S[4 * j + 1] * kk[j].y;
@@ -370,18 +392,25 @@ gated_delta_rule_reg_kernel(RecArgs a, const float *__restrict__ qkv, int conv_s
             float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
 #pragma unroll
             for (int j = 0; j < RP / 4; ++j) {
-                const float4 qq = q4[REG_LANES * j];
                 S[4 * j] = g * S[4 * j] + kk[j].x * u;
                 S[4 * j + 1] = g * S[4 * j + 1] + kk[j].y * u;
                 S[4 * j + 2] = g * S[4 * j + 2] + kk[j].z * u;
                 S[4 * j + 3] = g * S[4 * j + 3] + kk[j].w * u;
-                o0 += S[4 * j] * qq.x;
-                o1 += S[4 * j + 1] * qq.y;
-                o2 += S[4 * j + 2] * qq.z;
-                o3 += S[4 * j + 3] * qq.w;
+                o0 += S[4 * j] * qq[j].x;
+                o1 += S[4 * j + 1] * qq[j].y;
+                o2 += S[4 * j + 2] * qq[j].z;
+                o3 += S[4 * j + 3] * qq[j].w;
             }
             const float o = row16_sum((o0 + o1) + (o2 + o3)) * mq;
-            if (on && r == 0) a.out[(size_t)(q0 + t0 + tt) * a.heads * dv + head * dv + col] = o;
+            if (r == 0) os[tt * REG_BLOCK_COLS + wave * REG_COLS + c] = o;
+        }
+        __syncthreads();
+        // the chunk's read-outs leave together, 16 neighbouring columns a token
+#pragma unroll
+        for (int j = 0; j < VPER; ++j) {
+            const int x = tid + REG_THREADS * j, tt = x / REG_BLOCK_COLS, cc = x % REG_BLOCK_COLS;
+            if (tt < m && block_col0 + cc < dv)
+                a.out[(size_t)(q0 + t0 + tt) * a.heads * dv + head * dv + block_col0 + cc] = os[x];
         }
     }
     if (on)
@@ -400,7 +429,7 @@ gated_linear_attention_reg_kernel(RecArgs a, const void *__restrict__ y, int y_d
     __shared__ __attribute__((aligned(16))) float qs[CH * DS];
     __shared__ __attribute__((aligned(16))) float ks[CH * DS];
     __shared__ __attribute__((aligned(16))) float as[CH * DS];
-    __shared__ float vs[CH * REG_BLOCK_COLS];
+    __shared__ float vs[CH * REG_BLOCK_COLS], os[CH * REG_BLOCK_COLS];
     const int tid = threadIdx.x, lane = tid % KVA_WAVE, wave = tid / KVA_WAVE;
     const int c = lane / REG_LANES, r = lane % REG_LANES;
     const int slices = (a.vdim + REG_BLOCK_COLS - 1) / REG_BLOCK_COLS;
@@ -418,7 +447,8 @@ gated_linear_attention_reg_kernel(RecArgs a, const void *__restrict__ y, int y_d
         const int i = 4 * (REG_LANES * (j / 4) + r) + j % 4;
         S[j] = (on && i < d) ? Sg[(size_t)i * dv + col] : 0.f;
     }
-    float pq[PER], pk[PER], pa[PER], pv = 0.f;
+    constexpr int VPER = CH * REG_BLOCK_COLS / REG_THREADS;
+    float pq[PER], pk[PER], pa[PER], pv[VPER];
     auto fetch = [&](int t0, int m) {
 #pragma unroll
         for (int j = 0; j < PER; ++j) {
@@ -431,9 +461,12 @@ gated_linear_attention_reg_kernel(RecArgs a, const void *__restrict__ y, int y_d
             pk[j] = rec_ld(y, y_dtype, row * y_stride + k_off + head * d + i);
             pa[j] = alpha[row * alpha_stride + head * d + i];
         }
-        const int tt = tid / REG_BLOCK_COLS, cc = tid % REG_BLOCK_COLS;
-        pv = (tt < m && block_col0 + cc < dv)
-                 ? rec_ld(y, y_dtype, (size_t)(q0 + t0 + tt) * y_stride + v_off + head * dv + block_col0 + cc) : 0.f;
+#pragma unroll
+        for (int j = 0; j < VPER; ++j) {   // the chunk's tokens x 16 columns
+            const int x = tid + REG_THREADS * j, tt = x / REG_BLOCK_COLS, cc = x % REG_BLOCK_COLS;
+            pv[j] = (tt < m && block_col0 + cc < dv)
+                        ? rec_ld(y, y_dtype, (size_t)(q0 + t0 + tt) * y_stride + v_off + head * dv + block_col0 + cc) : 0.f;
+        }
     };
     fetch(0, min(CH, n));
     for (int t0 = 0; t0 < n; t0 += CH) {
@@ -446,29 +479,60 @@ gated_linear_attention_reg_kernel(RecArgs a, const void *__restrict__ y, int y_d
             ks[at] = pk[j];
             as[at] = pa[j];
         }
-        vs[tid] = pv;
+#pragma unroll
+        for (int j = 0; j < VPER; ++j) vs[tid + REG_THREADS * j] = pv[j];
         __syncthreads();
         if (t0 + CH < n) fetch(t0 + CH, min(CH, n - t0 - CH));
-        for (int tt = 0; tt < m; ++tt) {
+        // a token's operands are read from LDS into registers while the token before it is worked on
+        float4 kn[RP / 4], qn[RP / 4], an[RP / 4];
+        float vn;
+        auto read_token = [&](int tt) {
             const float4 *k4 = reinterpret_cast<const float4 *>(ks + tt * DS) + r;
             const float4 *q4 = reinterpret_cast<const float4 *>(qs + tt * DS) + r;
             const float4 *a4 = reinterpret_cast<const float4 *>(as + tt * DS) + r;
-            const float v = vs[tt * REG_BLOCK_COLS + wave * REG_COLS + c];
+#pragma unroll
+            for (int j = 0; j < RP / 4; ++j) {
+                kn[j] = k4[REG_LANES * j];
+                qn[j] = q4[REG_LANES * j];
+                an[j] = a4[REG_LANES * j];
+            }
+            vn = vs[tt * REG_BLOCK_COLS + wave * REG_COLS + c];
+        };
+        read_token(0);
+        // (unrolled: a token's sums over the rows and its write overlap the next token's update of S)
+#pragma unroll 4
+        for (int tt = 0; tt < m; ++tt) {
+            float4 kk[RP / 4], qq[RP / 4], al[RP / 4];
+            const float v = vn;
+#pragma unroll
+            for (int j = 0; j < RP / 4; ++j) {
+                kk[j] = kn[j];
+                qq[j] = qn[j];
+                al[j] = an[j];
+            }
+            read_token(min(tt + 1, CH - 1));
             float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
 #pragma unroll
             for (int j = 0; j < RP / 4; ++j) {
-                const float4 kk = k4[REG_LANES * j], qq = q4[REG_LANES * j], al = a4[REG_LANES * j];
-                S[4 * j] = al.x * S[4 * j] + kk.x * v;
-                S[4 * j + 1] = al.y * S[4 * j + 1] + kk.y * v;
-                S[4 * j + 2] = al.z * S[4 * j + 2] + kk.z * v;
-                S[4 * j + 3] = al.w * S[4 * j + 3] + kk.w * v;
-                o0 += S[4 * j] * qq.x;
-                o1 += S[4 * j + 1] * qq.y;
-                o2 += S[4 * j + 2] * qq.z;
-                o3 += S[4 * j + 3] * qq.w;
+                S[4 * j] = al[j].x * S[4 * j] + kk[j].x * v;
+                S[4 * j + 1] = al[j].y * S[4 * j + 1] + kk[j].y * v;
+                S[4 * j + 2] = al[j].z * S[4 * j + 2] + kk[j].z * v;
+                S[4 * j + 3] = al[j].w * S[4 * j + 3] + kk[j].w * v;
+                o0 += S[4 * j] * qq[j].x;
+                o1 += S[4 * j + 1] * qq[j].y;
+                o2 += S[4 * j + 2] * qq[j].z;
+                o3 += S[4 * j + 3] * qq[j].w;
             }
             const float o = row16_sum((o0 + o1) + (o2 + o3));
-            if (on && r == 0) a.out[(size_t)(q0 + t0 + tt) * a.heads * dv + head * dv + col] = o;
+            if (r == 0) os[tt * REG_BLOCK_COLS + wave * REG_COLS + c] = o;
+        }
+        __syncthreads();
+        // the chunk's read-outs leave together, 16 neighbouring columns a token
+#pragma unroll
+        for (int j = 0; j < VPER; ++j) {
+            const int x = tid + REG_THREADS * j, tt = x / REG_BLOCK_COLS, cc = x % REG_BLOCK_COLS;
+            if (tt < m && block_col0 + cc < dv)
+                a.out[(size_t)(q0 + t0 + tt) * a.heads * dv + head * dv + block_col0 + cc] = os[x];
         }
     }
     if (on)
