@@ -93,14 +93,18 @@ def gadopel_config(layers: int, vocab: int) -> dict:
 # linear attention with 16 heads of 64 x 128; every layer has 16 routed experts of width 1,024 and 2
 # identity experts, 4 choices a token (67 M expert weights a layer against the Llama layer's 50 M of
 # feed-forward; a token uses a quarter of them).
-def radilix_config(layers: int, vocab: int) -> dict:
-    mlp = {"kind": "moe", "expert": {"ff": 1024}, "router": {"experts": 16, "identity": 2, "top": 4}}
+# At another --width W the head counts and the experts' width scale with it (W / 64 attention heads over
+# W / 256 kv heads, W / 256 delta-rule heads, W / 128 heads of gated linear attention, experts of W / 2).
+def radilix_config(layers: int, vocab: int, width: int = 2048) -> dict:
+    W = width
+    mlp = {"kind": "moe", "expert": {"ff": W // 2}, "router": {"experts": 16, "identity": 2, "top": 4}}
     side = {"type": "parallel", "mlp": mlp, "mixer": {
-        "left": {"heads": 32, "kv_heads": 8, "dim": 64, "vdim": 64, "scale": 0.125, "rot": {"base": 500000.0, "dims": 32}},
-        "right": {"heads": 8, "kv_heads": 4, "dim": 128, "vdim": 128, "conv": 4},
+        "left": {"heads": W // 64, "kv_heads": W // 256, "dim": 64, "vdim": 64, "scale": 0.125,
+                 "rot": {"base": 500000.0, "dims": 32}},
+        "right": {"heads": W // 256, "kv_heads": W // 512, "dim": 128, "vdim": 128, "conv": 4},
         "left_scale": 1.0, "right_scale": 0.5}}
-    gla = {"type": "gla", "mlp": mlp, "mixer": {"heads": 16, "dim": 64, "vdim": 128, "tau": 16.0, "decay_rank": 16}}
-    return {"architecture": "Radilix", "vocab": vocab, "width": 2048, "norm": {"eps": 1e-6}, "residual_mult": 0.7,
+    gla = {"type": "gla", "mlp": mlp, "mixer": {"heads": W // 128, "dim": 64, "vdim": 128, "tau": 16.0, "decay_rank": 16}}
+    return {"architecture": "Radilix", "vocab": vocab, "width": W, "norm": {"eps": 1e-6}, "residual_mult": 0.7,
             "layers": [gla if i % 4 == 3 else side for i in range(layers)], "max_positions": 8192}
 
 
@@ -112,8 +116,17 @@ def design_comparison(args) -> int:
 
     layers, vocab = args.layers or 8, 32000
     llama = dict(CONFIG_1B, num_hidden_layers=layers, vocab_size=vocab, tie_word_embeddings=False)
-    design = args.design
-    configs = {design: {"gadopel": gadopel_config, "radilix": radilix_config}[design](layers, vocab), "llama": llama}
+    design, width = args.design, args.width
+    if width != 2048:
+        if design != "radilix" or width % 512 or not 512 <= width <= 8192:
+            print("--width: a multiple of 512 from 512 to 8192, for --design radilix")
+            return 2
+        llama.update(hidden_size=width, intermediate_size=4 * width, num_attention_heads=width // 64,
+                     num_key_value_heads=width // 256)
+        made = radilix_config(layers, vocab, width)
+    else:
+        made = {"gadopel": gadopel_config, "radilix": radilix_config}[design](layers, vocab)
+    configs = {design: made, "llama": llama}
     shapes = [(8, 4096), (32, 2048)]            # (requests, context) of the decode runs
     gen = torch.Generator().manual_seed(0)
     out = {}
@@ -189,7 +202,7 @@ def design_comparison(args) -> int:
     print(json.dumps({"metric": f"{design}_decode_tokens_per_second", "value": out[design][f"decode_b{b}_c{c}_tok_s"],
                       "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
                       "higher_is_better": True, "dtype": "bf16", "data": "synthetic (random weights, seeded token ids)",
-                      "config": {"design": f"{design} beside llama", "layers": layers, "width": 2048, "ff": 8192,
+                      "config": {"design": f"{design} beside llama", "layers": layers, "width": width, "ff": 4 * width,
                                  "vocab": vocab, "decode_shapes": shapes, "prefill_tokens": PREFILL_TOKENS},
                       "designs": out}))
     return 0
@@ -200,6 +213,8 @@ def main():
     ap.add_argument("--design", choices=["gadopel", "radilix"], default=None,
                     help="another measurement (its own JSON line): a model of this design at the layer sizes of a "
                          "served model beside a Llama model of equal size; the default run is left as it is")
+    ap.add_argument("--width", type=int, default=2048, help="--design radilix: the models' width (head counts and "
+                    "feed-forward sizes scale with it)")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=16)
