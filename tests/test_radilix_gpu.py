@@ -223,3 +223,44 @@ def test_contiguous_cache_mode_gives_the_logits_of_the_plain_model(dtype, models
     reqs = {f"c{i}": U.prompt(cfg, n, 90 + i) for i, n in enumerate([70, 33, 121])}
     eng = engine_for(folder, dtype, cache_mode="contiguous", cache_tokens=4 * 128, max_seq_len=128)
     check(eng, cfg, state, reqs, R.mixed(reqs, seed=9, max_live=3), dtype, "contiguous")
+
+
+def test_the_serving_process_serves_the_model_in_both_cache_modes(models, tmp_path, gpu):
+    """``cli.client`` starts ``cli.serve`` on the model folder: every sequence emits its budget and
+    the paged and the contiguous cache emit the same ids (scheduler, sampler and command line are the
+    ones every architecture uses)."""
+    import json
+    import os
+    import subprocess
+    import sys
+    cfg, folder, state = models["A"]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    results = {}
+    for mode in ("paged", "contiguous"):
+        out = tmp_path / f"{mode}.json"
+        env = dict(os.environ, IGNORE_EOS="1", ORCA_POLICY="oracle", PYTHONPATH=root)
+        cmd = [sys.executable, "-m", "kv_cache_optimization_for_llm_amd.cli.client", folder, "5", "--prompt-len", "37",
+               "--max-new-tokens", "10", "--num-seqs", "2", "--out", str(out), "--", "--dtype", "float32",
+               "--cache-mode", mode, "--max-seqs", "4", "--max-seq-len", "64", "--cache-tokens", "384",
+               "--chunk-size", "8", "--max-batch-tokens", "24"]
+        proc = subprocess.run(cmd, env=env, cwd=root, capture_output=True, text=True, timeout=280)
+        assert proc.returncode == 0, proc.stdout + proc.stderr
+        results[mode] = json.load(open(out))
+    for r in results.values():
+        assert r["status"] == "ok" and r["sequences_done"] == 10 and r["tokens"] == 100
+        assert r["count_mismatches"] == 0 and r["budget_mismatches"] == 0 and r["errors"] == []
+    assert results["paged"]["checksums"] == results["contiguous"]["checksums"]
+
+
+def test_the_sweep_command_runs_a_configuration_file_of_this_architecture(models, tmp_path, gpu):
+    import json
+    import os
+    from kv_cache_optimization_for_llm_amd.cli import sweep
+    cfg, folder, state = models["C"]
+    out = tmp_path / "sweep.jsonl"
+    assert sweep.main(["--shapes", os.path.join(folder, "config.json"), "--batches", "3", "--cache-modes", "paged",
+                       "--prompt-len", "40", "--prompt-min", "5", "--workload", "mixed", "--new-tokens", "9",
+                       "--max-seqs", "2", "--out", str(out)]) == 0
+    line, = [json.loads(l) for l in out.read_text().splitlines()]
+    assert line["requests_done"] == 3 and line["tokens_emitted"] == 27 and line["finish_reasons"] == {"length": 3}
+    assert line["layers"] == 5 and line["pages_reused"] > 0

@@ -63,7 +63,8 @@ def test_router_takes_the_lowest_index_of_equal_scores(gpu):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("width, ff, experts, identity, top, tokens",
                          [(64, 32, 4, 1, 2, 1), (64, 96, 7, 2, 3, 50), (72, 40, 3, 0, 3, 33), (96, 48, 1, 4, 2, 17),
-                          (128, 160, 16, 2, 4, 300), (40, 24, 2, 2, 4, 9)])
+                          (128, 160, 16, 2, 4, 300), (40, 24, 2, 2, 4, 9),
+                          (64, 1024, 4, 1, 2, 1200), (1024, 96, 3, 0, 2, 1500)])      # many tiles: row tiles that share an expert's matrix
 def test_routed_experts_against_the_plain_mixture(width, ff, experts, identity, top, tokens, dtype, gpu):
     from kv_cache_optimization_for_llm_amd.parts.base import MixerContext
     from kv_cache_optimization_for_llm_amd.parts.moe import RoutedExperts
