@@ -142,10 +142,10 @@ def run_in_steps(lengths, portions_of, launch):
 
 
 @pytest.mark.parametrize("heads, kv_heads, dim, vdim", [(2, 1, 32, 32), (4, 2, 16, 24), (3, 3, 20, 7), (2, 2, 128, 48), (6, 2, 8, 70), (2, 1, 160, 20), (1, 1, 64, 3)])
-@pytest.mark.parametrize("portions", [(1000,), (1,), (2, 1, 17, 5, 64)])
+@pytest.mark.parametrize("portions", [(1000,), (1,), (2, 1, 17, 5, 64), (32, 31, 1, 33)])     # the last: cuts at the kernels' chunk of 32 tokens
 def test_gated_delta_rule_over_steps(heads, kv_heads, dim, vdim, portions, gpu):
     g = torch.Generator().manual_seed(heads * dim + vdim)
-    lengths = {2: 75, 0: 9, 1: 40}
+    lengths = {2: 131, 0: 9, 1: 64}
     C = 2 * kv_heads * dim + heads * vdim
     ycols, boff, doff = 2 * heads + 3, 1, heads + 2
     qkv = {s: torch.randn(n, C, generator=g) for s, n in lengths.items()}
@@ -178,10 +178,10 @@ def test_gated_delta_rule_over_steps(heads, kv_heads, dim, vdim, portions, gpu):
 
 
 @pytest.mark.parametrize("heads, dim, vdim", [(4, 48, 32), (1, 16, 16), (3, 20, 9), (2, 128, 40), (5, 8, 64), (2, 144, 18), (1, 100, 5)])
-@pytest.mark.parametrize("portions", [(1000,), (1,), (3, 1, 16, 2, 50)])
+@pytest.mark.parametrize("portions", [(1000,), (1,), (3, 1, 16, 2, 50), (31, 33, 32, 1)])
 def test_gated_linear_attention_over_steps(heads, dim, vdim, portions, gpu):
     g = torch.Generator().manual_seed(heads * dim + vdim + 1)
-    lengths = {1: 66, 0: 5, 2: 31}
+    lengths = {1: 97, 0: 5, 2: 32}
     q_off, k_off, v_off = 3, 3 + heads * dim, 3 + 2 * heads * dim
     ycols = v_off + heads * vdim + 2
     y = {s: torch.randn(n, ycols, generator=g) for s, n in lengths.items()}
