@@ -265,6 +265,30 @@ gated_linear_attention_kernel(RecArgs a, const void *__restrict__ y, int y_dtype
 #define REG_BLOCK_COLS (REG_COLS * REG_WAVES)
 #define REG_THREADS (KVA_WAVE * REG_WAVES)
 
+// Sums over the 16 lanes of a row for several values at once, stage by stage: the rotations of one
+// value do not wait for each other's results but stand between those of the others (a dependent
+// instruction of a wavefront that has its SIMD to itself waits some 16 cycles for its operand).
+template <int N>
+__device__ inline void row16_sum_each(float (&x)[N]) {
+    float t[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) t[i] = row16_rotated<8>(x[i]);
+#pragma unroll
+    for (int i = 0; i < N; ++i) x[i] += t[i];
+#pragma unroll
+    for (int i = 0; i < N; ++i) t[i] = row16_rotated<4>(x[i]);
+#pragma unroll
+    for (int i = 0; i < N; ++i) x[i] += t[i];
+#pragma unroll
+    for (int i = 0; i < N; ++i) t[i] = row16_rotated<2>(x[i]);
+#pragma unroll
+    for (int i = 0; i < N; ++i) x[i] += t[i];
+#pragma unroll
+    for (int i = 0; i < N; ++i) t[i] = row16_rotated<1>(x[i]);
+#pragma unroll
+    for (int i = 0; i < N; ++i) x[i] += t[i];
+}
+
 template <int RP>
 __global__ void __launch_bounds__(REG_THREADS)
 gated_delta_rule_reg_kernel(RecArgs a, const float *__restrict__ qkv, int conv_stride, const void *__restrict__ y,
@@ -352,57 +376,52 @@ gated_delta_rule_reg_kernel(RecArgs a, const float *__restrict__ qkv, int conv_s
         }
         __syncthreads();
         if (t0 + CH < n) fetch(t0 + CH, min(CH, n - t0 - CH));
-        // a token's operands are read from LDS into registers while the token before it is worked on
-        float4 kn[RP / 4], qn[RP / 4];
-        float gn, betan, vn, mqn, mkn;
-        auto read_token = [&](int tt) {
-            const float4 *k4 = reinterpret_cast<const float4 *>(ks + tt * DS) + r;
-            const float4 *q4 = reinterpret_cast<const float4 *>(qs + tt * DS) + r;
+        // The walk.  Both sums over the rows that a token needs read the same S - the state before the
+        // token for S^T k, the state after it for S^T q - so the read-out of a token rides with the next
+        // token's S^T k: one pass over S, the two sums reduced side by side, and only the chain
+        // S^T k -> u -> S is what a token waits for.
+        float4 qp[RP / 4];                       // q of the token before (zero in front of the chunk's first)
+        float mqp = 0.f;
 #pragma unroll
-            for (int j = 0; j < RP / 4; ++j) {
-                kn[j] = k4[REG_LANES * j];
-                qn[j] = q4[REG_LANES * j];
-            }
-            gn = gs[tt]; betan = bs[tt]; vn = vs[tt * REG_BLOCK_COLS + wave * REG_COLS + c]; mqn = nq[tt]; mkn = nk[tt];
-        };
-        read_token(0);
-        // (unrolled: a token's sums over the rows and its write overlap the next token's update of S)
-#pragma unroll 4
-        for (int tt = 0; tt < m; ++tt) {
+        for (int j = 0; j < RP / 4; ++j) qp[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int tt = 0; tt <= m; ++tt) {
+            const bool last = tt == m;           // behind the chunk's last token only its read-out is left
+            const int at = min(tt, CH - 1);
+            const float4 *k4 = reinterpret_cast<const float4 *>(ks + at * DS) + r;
+            const float4 *q4 = reinterpret_cast<const float4 *>(qs + at * DS) + r;
+            const float g = gs[at], beta = bs[at], v = vs[at * REG_BLOCK_COLS + wave * REG_COLS + c], mq = nq[at], mk = nk[at];
             float4 kk[RP / 4], qq[RP / 4];
-            const float g = gn, beta = betan, v = vn, mq = mqn, mk = mkn;
+            float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f, p0 = 0.f, p1 = 0.f, p2 = 0.f, p3 = 0.f;
 #pragma unroll
             for (int j = 0; j < RP / 4; ++j) {
-                kk[j] = kn[j];
-                qq[j] = qn[j];
-            }
-            read_token(min(tt + 1, CH - 1));
-            // the unit vectors' factors multiply the sums: S^T (mk k) = mk (S^T k), S^T (mq q) likewise
-            float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
-#pragma unroll
-            for (int j = 0; j < RP / 4; ++j) {
+                kk[j] = k4[REG_LANES * j];
+                qq[j] = q4[REG_LANES * j];
+                // the unit vectors' factors multiply the sums: S^T (mk k) = mk (S^T k), S^T (mq q) likewise
                 kk[j].x *= mk; kk[j].y *= mk; kk[j].z *= mk; kk[j].w *= mk;
                 d0 += S[4 * j] * kk[j].x;
+                p0 += S[4 * j] * qp[j].x;
                 d1 += S[4 * j + 1] * kk[j].y;
+                p1 += S[4 * j + 1] * qp[j].y;
                 d2 += S[4 * j + 2] * kk[j].z;
+                p2 += S[4 * j + 2] * qp[j].z;
                 d3 += S[4 * j + 3] * kk[j].w;
+                p3 += S[4 * j + 3] * qp[j].w;
             }
-            const float dot = row16_sum((d0 + d1) + (d2 + d3));
-            const float u = beta * (v - g * dot);
-            float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
+            d0 += d1; p0 += p1; d2 += d3; p2 += p3;
+            float both[2] = {d0 + d2, p0 + p2};
+            row16_sum_each<2>(both);
+            if (tt > 0 && r == 0) os[(tt - 1) * REG_BLOCK_COLS + wave * REG_COLS + c] = both[1] * mqp;
+            if (last) break;
+            const float u = beta * (v - g * both[0]);
 #pragma unroll
             for (int j = 0; j < RP / 4; ++j) {
                 S[4 * j] = g * S[4 * j] + kk[j].x * u;
                 S[4 * j + 1] = g * S[4 * j + 1] + kk[j].y * u;
                 S[4 * j + 2] = g * S[4 * j + 2] + kk[j].z * u;
                 S[4 * j + 3] = g * S[4 * j + 3] + kk[j].w * u;
-                o0 += S[4 * j] * qq[j].x;
-                o1 += S[4 * j + 1] * qq[j].y;
-                o2 += S[4 * j + 2] * qq[j].z;
-                o3 += S[4 * j + 3] * qq[j].w;
+                qp[j] = qq[j];
             }
-            const float o = row16_sum((o0 + o1) + (o2 + o3)) * mq;
-            if (r == 0) os[tt * REG_BLOCK_COLS + wave * REG_COLS + c] = o;
+            mqp = mq;
         }
         __syncthreads();
         // the chunk's read-outs leave together, 16 neighbouring columns a token
@@ -483,48 +502,47 @@ gated_linear_attention_reg_kernel(RecArgs a, const void *__restrict__ y, int y_d
         for (int j = 0; j < VPER; ++j) vs[tid + REG_THREADS * j] = pv[j];
         __syncthreads();
         if (t0 + CH < n) fetch(t0 + CH, min(CH, n - t0 - CH));
-        // a token's operands are read from LDS into registers while the token before it is worked on
-        float4 kn[RP / 4], qn[RP / 4], an[RP / 4];
-        float vn;
-        auto read_token = [&](int tt) {
+        // The walk, four tokens at a time: only S is handed from token to token (two operations an
+        // element); the four read-outs' sums over the rows are independent of each other and are
+        // formed side by side, stage by stage.
+        auto step = [&](int tt, float (&o)[4]) {
             const float4 *k4 = reinterpret_cast<const float4 *>(ks + tt * DS) + r;
             const float4 *q4 = reinterpret_cast<const float4 *>(qs + tt * DS) + r;
             const float4 *a4 = reinterpret_cast<const float4 *>(as + tt * DS) + r;
+            const float v = vs[tt * REG_BLOCK_COLS + wave * REG_COLS + c];
+            o[0] = o[1] = o[2] = o[3] = 0.f;
 #pragma unroll
             for (int j = 0; j < RP / 4; ++j) {
-                kn[j] = k4[REG_LANES * j];
-                qn[j] = q4[REG_LANES * j];
-                an[j] = a4[REG_LANES * j];
+                const float4 kk = k4[REG_LANES * j], qq = q4[REG_LANES * j], al = a4[REG_LANES * j];
+                S[4 * j] = al.x * S[4 * j] + kk.x * v;
+                S[4 * j + 1] = al.y * S[4 * j + 1] + kk.y * v;
+                S[4 * j + 2] = al.z * S[4 * j + 2] + kk.z * v;
+                S[4 * j + 3] = al.w * S[4 * j + 3] + kk.w * v;
+                o[0] += S[4 * j] * qq.x;
+                o[1] += S[4 * j + 1] * qq.y;
+                o[2] += S[4 * j + 2] * qq.z;
+                o[3] += S[4 * j + 3] * qq.w;
             }
-            vn = vs[tt * REG_BLOCK_COLS + wave * REG_COLS + c];
         };
-        read_token(0);
-        // (unrolled: a token's sums over the rows and its write overlap the next token's update of S)
-#pragma unroll 4
-        for (int tt = 0; tt < m; ++tt) {
-            float4 kk[RP / 4], qq[RP / 4], al[RP / 4];
-            const float v = vn;
+        int tt = 0;
+        for (; tt + 4 <= m; tt += 4) {
+            float o[4][4], sum[4];
 #pragma unroll
-            for (int j = 0; j < RP / 4; ++j) {
-                kk[j] = kn[j];
-                qq[j] = qn[j];
-                al[j] = an[j];
-            }
-            read_token(min(tt + 1, CH - 1));
-            float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
+            for (int i = 0; i < 4; ++i) step(tt + i, o[i]);
 #pragma unroll
-            for (int j = 0; j < RP / 4; ++j) {
-                S[4 * j] = al[j].x * S[4 * j] + kk[j].x * v;
-                S[4 * j + 1] = al[j].y * S[4 * j + 1] + kk[j].y * v;
-                S[4 * j + 2] = al[j].z * S[4 * j + 2] + kk[j].z * v;
-                S[4 * j + 3] = al[j].w * S[4 * j + 3] + kk[j].w * v;
-                o0 += S[4 * j] * qq[j].x;
-                o1 += S[4 * j + 1] * qq[j].y;
-                o2 += S[4 * j + 2] * qq[j].z;
-                o3 += S[4 * j + 3] * qq[j].w;
-            }
-            const float o = row16_sum((o0 + o1) + (o2 + o3));
-            if (r == 0) os[tt * REG_BLOCK_COLS + wave * REG_COLS + c] = o;
+            for (int i = 0; i < 4; ++i) { o[i][0] += o[i][1]; o[i][2] += o[i][3]; }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) sum[i] = o[i][0] + o[i][2];
+            row16_sum_each<4>(sum);
+            if (r == 0)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) os[(tt + i) * REG_BLOCK_COLS + wave * REG_COLS + c] = sum[i];
+        }
+        for (; tt < m; ++tt) {
+            float o[4];
+            step(tt, o);
+            const float sum = row16_sum((o[0] + o[1]) + (o[2] + o[3]));
+            if (r == 0) os[tt * REG_BLOCK_COLS + wave * REG_COLS + c] = sum;
         }
         __syncthreads();
         // the chunk's read-outs leave together, 16 neighbouring columns a token
